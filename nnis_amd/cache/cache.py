@@ -50,7 +50,7 @@ class KVGroup:
     def __init__(self, request: KVRequest, entries: List[int], pages: int, slots: int, max_positions: int,
                  dtype: torch.dtype, device):
         self.request = request
-        self.entries = entries  # schedule indices, in order
+        self.entries = entries  # who keeps a cache here (schedule entries, or places inside them), in order
         # a windowed group has storage and pages of its own; it keeps every
         # page of a sequence (the kernels mask by the window), so that a whole
         # prompt can be written before its scores are taken
@@ -109,9 +109,9 @@ class SequenceCache:
 
     def __init__(self, requests: Sequence[Tuple[int, Any]], shared: Dict[int, int], max_tokens: int, max_positions: int,
                  dtype: torch.dtype, device, max_slots: Optional[int] = None):
-        """``requests``: (schedule index, KVRequest | StateRequest | None) for
-        entries that keep a cache; ``shared``: schedule index -> index of the
-        entry whose cache it reads."""
+        """``requests``: (schedule index, KVRequest | StateRequest | None, or
+        a tuple of such) for entries that keep a cache; ``shared``: schedule
+        index -> index of the entry whose cache it reads."""
         if max_tokens <= 0:
             raise InvalidInput(f"max_tokens must be positive; got {max_tokens}")
         self.device = torch.device(device)
@@ -126,27 +126,63 @@ class SequenceCache:
         self.state_regions: Dict[str, torch.Tensor] = {}
         self._layer_state: List[str] = []  # regions that a mixer's StateRequest asked for
         self._views: Dict[int, Any] = {}
-        grouped: Dict[KVRequest, List[int]] = {}
-        for index, request in requests:
-            if isinstance(request, KVRequest):
-                grouped.setdefault(request, []).append(index)
-            elif isinstance(request, StateRequest):
-                region = self.add_state_region(f"entry{index}", request.shape, getattr(torch, request.dtype))
-                self._layer_state.append(f"entry{index}")
-                self._views[index] = StateView(region, read_only=False)
-            elif request is not None:
+        # A request is a KVRequest, a StateRequest, None, or a tuple of requests (a mixer made of several, or one
+        # that keeps more than one thing): its view is then the tuple of their views, in order.  ``places`` names
+        # every single request by (schedule entry, path inside the entry's tuples).
+        places: List[Tuple[Any, Tuple[int, ...], Any]] = []
+
+        def walk(index, path, request):
+            if isinstance(request, (tuple, list)):
+                for position, inner in enumerate(request):
+                    walk(index, path + (position,), inner)
+            elif isinstance(request, (KVRequest, StateRequest)) or request is None:
+                places.append((index, path, request))
+            else:
                 raise InvalidInput(f"schedule entry {index}: unknown cache request {request!r}")
+
+        for index, request in requests:
+            walk(index, (), request)
+        single: Dict[Tuple[Any, Tuple[int, ...]], Any] = {}
+        grouped: Dict[KVRequest, List[Tuple[Any, Tuple[int, ...]]]] = {}
+        for index, path, request in places:
+            if isinstance(request, KVRequest):
+                grouped.setdefault(request, []).append((index, path))
+            elif isinstance(request, StateRequest):
+                name = f"entry{index}" + "".join(f".{position}" for position in path)
+                region = self.add_state_region(name, request.shape, getattr(torch, request.dtype))
+                self._layer_state.append(name)
+                single[(index, path)] = StateView(region, read_only=False)
+            else:
+                single[(index, path)] = None
         for request, entries in grouped.items():
             group = KVGroup(request, entries, self.pages, self.max_slots, max_positions, dtype, self.device)
             self.kv_groups.append(group)
-            for position, index in enumerate(entries):
-                self._views[index] = KVView(group.k[position], group.v[position], group.block_table, request.window, False)
-        for index, owner in shared.items():
-            view = self._views.get(owner)
+            for position, place in enumerate(entries):
+                single[place] = KVView(group.k[position], group.v[position], group.block_table, request.window, False)
+
+        def gather(index, path, request):
+            if isinstance(request, (tuple, list)):
+                return tuple(gather(index, path + (position,), inner) for position, inner in enumerate(request))
+            return single[(index, path)]
+
+        for index, request in requests:
+            view = gather(index, (), request)
+            if view is not None:
+                self._views[index] = view
+
+        def shared_view(view):
+            if isinstance(view, tuple):
+                return tuple(shared_view(inner) for inner in view)
             if isinstance(view, KVView):
-                self._views[index] = KVView(view.k_pages, view.v_pages, view.block_table, view.window, True)
-            elif isinstance(view, StateView):
-                self._views[index] = StateView(view.state, True)
+                return KVView(view.k_pages, view.v_pages, view.block_table, view.window, True)
+            if isinstance(view, StateView):
+                return StateView(view.state, True)
+            return None
+
+        for index, owner in shared.items():
+            view = shared_view(self._views.get(owner))
+            if view is not None:
+                self._views[index] = view
 
     # ---- state regions ----------------------------------------------------
     def add_state_region(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:

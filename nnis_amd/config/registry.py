@@ -1,6 +1,7 @@
 """The one registry from an architecture's name to its model.
 
-``config.json`` names the architecture in ``architectures[0]``; the registry
+``config.json`` names the architecture in ``architectures[0]`` (or, as one
+name, in ``architecture``); the registry
 maps that name to a configuration class (``from_dict(raw) -> config``) and a
 builder (``config -> ModelSpec``).  The reference gates on the name with an
 ``if`` (/root/reference/crates/nnis-model/src/safetensors_loader.rs:137-145);
@@ -37,6 +38,8 @@ def registered_architectures() -> List[str]:
 
 def lookup_architecture(raw_config: Dict[str, Any]) -> Architecture:
     names = raw_config.get("architectures")
+    if names is None and isinstance(raw_config.get("architecture"), str):
+        names = [raw_config["architecture"]]
     if not isinstance(names, list) or len(names) != 1 or not isinstance(names[0], str):
         raise InvalidInput(f"config.json architectures must be a list with one name; got {names!r}")
     entry = _ARCHITECTURES.get(names[0])

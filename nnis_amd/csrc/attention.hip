@@ -35,11 +35,18 @@ extern "C" int nnis_attention_head_dim() { return NNIS_HEAD_DIM; }
 namespace {
 
 constexpr int HD = NNIS_HEAD_DIM;
+// channels of a value head: the keys' unless the module is compiled for values of another size
+#ifndef NNIS_VALUE_DIM
+#define NNIS_VALUE_DIM NNIS_HEAD_DIM
+#endif
+constexpr int HDV = NNIS_VALUE_DIM;
+// the matrix-core kernels below take heads in steps of 16 channels whose values are as wide as their keys
+#define NNIS_MATRIX_CORES (NNIS_HEAD_DIM % 16 == 0 && NNIS_VALUE_DIM == NNIS_HEAD_DIM)
 
 struct AttnArgs {
   const void* q;  // [tokens, heads, HD]
   int q_dtype;
-  void* out;  // [tokens, heads, HD]
+  void* out;  // [tokens, heads, HDV]
   int out_dtype;
   const void* k_pages;
   const void* v_pages;
@@ -51,6 +58,7 @@ struct AttnArgs {
   int tokens, heads, kv_heads;
   int window;  // 0: all keys
   float scale;
+  float softcap;  // 0: none; else a score s becomes softcap * tanh(s / softcap)
 };
 
 // One wave per (token, query head); lanes take keys lo+lane, lo+lane+64, ...,
@@ -65,9 +73,10 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   const int token = item / a.heads;
   const int head = item % a.heads;
   const size_t row = ((size_t)token * a.heads + head) * HD;
+  const size_t out_row = ((size_t)token * a.heads + head) * HDV;
   const int slot = a.tok_slot[token];
   if (slot < 0) {  // padding row
-    for (int d = lane; d < HD; d += kWave) store_from_f32(a.out, a.out_dtype, row + d, 0.0f);
+    for (int d = lane; d < HDV; d += kWave) store_from_f32(a.out, a.out_dtype, out_row + d, 0.0f);
     return;
   }
   const int pos = a.tok_pos[token];
@@ -85,9 +94,9 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   const int* pages = a.block_table + (size_t)slot * a.max_pages;
 
   float m = -INFINITY, l = 0.0f;
-  float o[HD];
+  float o[HDV];
 #pragma unroll
-  for (int d = 0; d < HD; ++d) o[d] = 0.0f;
+  for (int d = 0; d < HDV; ++d) o[d] = 0.0f;
 
   for (int j = lo + lane; j < kv_len; j += kWave) {
     const int page = pages[j / kPageTokens];
@@ -96,14 +105,15 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
     float dot = 0.0f;
 #pragma unroll
     for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_f32(keys[nnis_k_offset(r, d)]), dot);
-    const float s = dot * a.scale;
+    float s = dot * a.scale;
+    if (a.softcap > 0.0f) s = a.softcap * tanhf(s / a.softcap);
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first key
     const float p = expf(s - m_new);
     l = l * alpha + p;
-    const CacheT* values = vp + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
+    const CacheT* values = vp + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HDV);
 #pragma unroll
-    for (int d = 0; d < HD; ++d) o[d] = o[d] * alpha + p * to_f32(values[nnis_v_offset(d, r)]);
+    for (int d = 0; d < HDV; ++d) o[d] = o[d] * alpha + p * to_f32(values[nnis_v_offset(d, r)]);
     m = m_new;
   }
 
@@ -111,16 +121,16 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   const float factor = (m == -INFINITY) ? 0.0f : expf(m - m_all);
   const float l_all = wave_sum(l * factor);
   const float inv = 1.0f / l_all;
-  float mine[(HD + kWave - 1) / kWave];
+  float mine[(HDV + kWave - 1) / kWave];
 #pragma unroll
-  for (int d = 0; d < HD; ++d) {
+  for (int d = 0; d < HDV; ++d) {
     const float total = wave_sum(o[d] * factor);
     if (d % kWave == lane) mine[d / kWave] = total * inv;
   }
 #pragma unroll
-  for (int c = 0; c < (HD + kWave - 1) / kWave; ++c) {
+  for (int c = 0; c < (HDV + kWave - 1) / kWave; ++c) {
     const int d = c * kWave + lane;
-    if (d < HD) store_from_f32(a.out, a.out_dtype, row + d, mine[c]);
+    if (d < HDV) store_from_f32(a.out, a.out_dtype, out_row + d, mine[c]);
   }
 }
 
@@ -145,7 +155,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
 // scaled by log2 e); probabilities are rounded to bfloat16 for the product
 // with the bfloat16 values.
 // =============================================================================
-#if NNIS_HEAD_DIM % 16 == 0
+#if NNIS_MATRIX_CORES
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -1112,15 +1122,17 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
   }
 }
 
-#endif  // NNIS_HEAD_DIM % 16 == 0
+#endif  // NNIS_MATRIX_CORES
 
 }  // namespace
 
 extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
                                    const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
                                    const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
-                                   int head_dim, int window, float scale, void* stream) {
+                                   int head_dim, int window, float scale, int value_dim, float softcap, void* stream) {
   NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
+  NNIS_REQUIRE((value_dim <= 0 ? head_dim : value_dim) == HDV, "attention: this module is compiled for values of %d channels, got %d", HDV, value_dim);
+  NNIS_REQUIRE(softcap >= 0.0f, "attention: the cap of the scores must not be negative, got %g", (double)softcap);
   NNIS_REQUIRE(nnis_dtype_ok(q_dtype) && nnis_dtype_ok(out_dtype) && nnis_dtype_ok(cache_dtype),
                "attention: unknown dtype (q %d, out %d, cache %d)", q_dtype, out_dtype, cache_dtype);
   NNIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: %d heads do not divide into %d kv heads",
@@ -1131,7 +1143,7 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
   a.q = q; a.q_dtype = q_dtype; a.out = out; a.out_dtype = out_dtype;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype;
   a.block_table = block_table; a.max_pages = max_pages; a.tok_slot = tok_slot; a.tok_pos = tok_pos;
-  a.tokens = tokens; a.heads = heads; a.kv_heads = kv_heads; a.window = window; a.scale = scale;
+  a.tokens = tokens; a.heads = heads; a.kv_heads = kv_heads; a.window = window; a.scale = scale; a.softcap = softcap;
   const long long items = (long long)tokens * heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
   if (cache_dtype == NNIS_F32) {
@@ -1144,7 +1156,7 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
 }
 
 
-#if NNIS_HEAD_DIM % 16 == 0
+#if NNIS_MATRIX_CORES
 namespace {
 constexpr int kMaxColumns = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // column tiles a wave carries (registers)
 
@@ -1371,14 +1383,14 @@ extern "C" int nnis_attention_prefill_tile_rows(int, int, int) { return 0; }
 extern "C" int nnis_attention_prefill_max_waves(int, int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
                                            int, const int*, const int*, const int*, int, int, int, int, float, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }
 extern "C" int nnis_attention_combine(const float*, void*, const int*, int, int, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
                                           int, int, int, int, int, float, int, int, float*, int, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 #endif

@@ -299,6 +299,9 @@ struct RopeWriteArgs {
   const int* block_table;  // [slots][max_pages]
   int max_pages;
   int heads, kv_heads, head_dim;
+  int value_dim;     // channels of a value head (head_dim unless the values have a size of their own)
+  const void* bias;  // [(heads + kv_heads) * head_dim + kv_heads * value_dim] added before the rotation, or null
+  int bias_dtype;
 };
 
 __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
@@ -307,9 +310,15 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   if (slot < 0) return;
   const int pos = a.tok_pos[token];
   const int hd = a.head_dim;
+  const int vd = a.value_dim;
   const int half = a.rot_dim / 2;
-  const int row_width = (a.heads + 2 * a.kv_heads) * hd;
+  const int row_width = (a.heads + a.kv_heads) * hd + a.kv_heads * vd;
   const size_t in_base = (size_t)token * row_width;
+  // element `at` of the token's row, with its bias
+  auto element = [&](size_t at) {
+    const float v = load_as_f32(a.qkv, a.qkv_dtype, in_base + at);
+    return a.bias ? v + load_as_f32(a.bias, a.bias_dtype, at) : v;
+  };
   const bool rotate = a.cos_table != nullptr && pos < a.table_positions;
   const float* cos_row = rotate ? a.cos_table + (size_t)pos * half : nullptr;
   const float* sin_row = rotate ? a.sin_table + (size_t)pos * half : nullptr;
@@ -324,12 +333,12 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   for (int item = threadIdx.x; item < rot_heads * items_per_head; item += blockDim.x) {
     const int head = item / items_per_head;
     const int e = item % items_per_head;
-    const size_t src = in_base + (size_t)head * hd;
+    const size_t src = (size_t)head * hd;
     float lo, hi = 0.0f;
     int lo_index, hi_index = -1;
     if (e < half) {
-      const float x0 = load_as_f32(a.qkv, a.qkv_dtype, src + e);
-      const float x1 = load_as_f32(a.qkv, a.qkv_dtype, src + e + half);
+      const float x0 = element(src + e);
+      const float x1 = element(src + e + half);
       float c = 1.0f, s = 0.0f;
       if (rotate) {
         c = cos_row[e];
@@ -341,7 +350,7 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
       hi_index = e + half;
     } else {
       lo_index = e + half;  // element index in [rot_dim, head_dim)
-      lo = load_as_f32(a.qkv, a.qkv_dtype, src + lo_index);
+      lo = element(src + lo_index);
     }
     if (head < a.heads) {
       const size_t dst = ((size_t)token * a.heads + head) * hd;
@@ -356,12 +365,12 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   }
   // values: copied into the page's order
   if (page >= 0) {
-    const size_t v_src = in_base + (size_t)(a.heads + a.kv_heads) * hd;
-    for (int item = threadIdx.x; item < a.kv_heads * hd; item += blockDim.x) {
-      const int kv_head = item / hd;
-      const int d = item % hd;
-      const float v = load_as_f32(a.qkv, a.qkv_dtype, v_src + item);
-      const size_t dst = ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(hd) + nnis_v_offset(d, in_page);
+    const size_t v_src = (size_t)(a.heads + a.kv_heads) * hd;
+    for (int item = threadIdx.x; item < a.kv_heads * vd; item += blockDim.x) {
+      const int kv_head = item / vd;
+      const int d = item % vd;
+      const float v = element(v_src + item);
+      const size_t dst = ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(vd) + nnis_v_offset(d, in_page);
       store_from_f32(a.v_pages, a.cache_dtype, dst, v);
     }
   }
@@ -432,11 +441,14 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
   }
 }
 
-extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
-                                  const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
-                                  const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
-                                  const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
-                                  int head_dim, void* stream) {
+// value_dim: channels of a value head (0: head_dim); bias: one entry per column of qkv, added before the rotation, or null
+extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
+                                       const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
+                                       const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
+                                       const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
+                                       int head_dim, int value_dim, const void* bias, int bias_dtype, void* stream) {
+  if (value_dim <= 0) value_dim = head_dim;
+  NNIS_REQUIRE(bias == nullptr || nnis_dtype_ok(bias_dtype), "rope_kv_write: unknown bias dtype %d", bias_dtype);
   NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype) && nnis_dtype_ok(q_dtype), "rope_kv_write: unknown dtype");
   NNIS_REQUIRE(k_pages == nullptr || nnis_dtype_ok(cache_dtype), "rope_kv_write: unknown cache dtype %d", cache_dtype);
   NNIS_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
@@ -453,21 +465,32 @@ extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, i
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.k_pages = k_pages; a.v_pages = v_pages;
   a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  a.value_dim = value_dim; a.bias = bias; a.bias_dtype = bias_dtype;
   const bool all_bf16 = qkv_dtype == NNIS_BF16 && q_dtype == NNIS_BF16 && (k_pages == nullptr || cache_dtype == NNIS_BF16);
   const bool aligned = ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)q_out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
                        ((uintptr_t)v_pages % 16 == 0) && ((uintptr_t)cos_table % 16 == 0) && ((uintptr_t)sin_table % 16 == 0);
-  if (all_bf16 && aligned && head_dim % 4 == 0 && (a.rot_dim / 2) % 4 == 0) {
+  if (all_bf16 && aligned && head_dim % 4 == 0 && (a.rot_dim / 2) % 4 == 0 && value_dim == head_dim && bias == nullptr) {
     const int items = (heads + kv_heads) * (head_dim - a.rot_dim / 2) / 4 + kv_heads * head_dim / 4;
     const int threads = items > 128 ? 256 : (items > 64 ? 128 : 64);
     hipLaunchKernelGGL(rope_kv_write_bf16_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
     NNIS_LAUNCH_CHECK("rope_kv_write_bf16");
     return 0;
   }
-  const int work = (heads + 2 * kv_heads) * head_dim / 2;
+  const int work = ((heads + kv_heads) * head_dim + kv_heads * value_dim) / 2;
   const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
   hipLaunchKernelGGL(rope_kv_write_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("rope_kv_write");
   return 0;
+}
+
+extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
+                                  const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
+                                  const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
+                                  const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
+                                  int head_dim, void* stream) {
+  return nnis_rope_kv_write_wide(qkv, qkv_dtype, q_out, q_dtype, cos_table, sin_table, table_positions, rot_dim, tok_slot, tok_pos,
+                                 k_pages, v_pages, cache_dtype, block_table, max_pages, tokens, heads, kv_heads, head_dim, 0,
+                                 nullptr, 0, stream);
 }
 
 // -----------------------------------------------------------------------------

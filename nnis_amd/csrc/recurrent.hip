@@ -1,0 +1,392 @@
+// Mixers that carry a state of fixed size from token to token: a short causal convolution per channel, the
+// selective scan (a diagonal recurrence per channel with input-dependent steps), gated linear attention (a
+// matrix state per head with a decay per key channel), and the per-head norm and gate behind it.
+//
+// A step's rows are packed: sequence b of the step owns rows seq_start[b] .. seq_start[b + 1] - 1, which
+// continue the sequence in slot seq_slot[b] (negative: padding, nothing is read or written for it).  State
+// lives per slot in 32-bit and is zero when a sequence starts; a kernel reads it at a run's first row and
+// leaves it behind the run's last, so a prompt in one step, in portions, or token by token give the same.
+// Decays, step sizes, exponentials and the recurrences themselves are 32-bit whatever the storage type.
+#include "common.h"
+
+thread_local char g_nnis_error[512] = {0};
+extern "C" const char* nnis_last_error() { return g_nnis_error; }
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+// log(sigmoid(z)) = min(z, 0) - log(1 + exp(-|z|))
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
+
+// -----------------------------------------------------------------------------
+// Causal convolution per channel with SiLU: y[t, c] = silu(b[c] + sum_j w[c, j] x[t - (taps - 1) + j, c]),
+// the last tap on the token itself, zeros before the sequence's start.  Inputs older than the step's first
+// row come from `state` [slots, taps - 1, channels] (the sequence's last taps - 1 inputs, oldest first).
+// -----------------------------------------------------------------------------
+constexpr int kMostTaps = 16;
+
+struct ConvArgs {
+  const void* x;  // [tokens, x_stride]: the first `channels` columns
+  int x_dtype;
+  int x_stride;
+  const void* weight;  // [channels, taps]
+  const void* bias;    // [channels] or null
+  int weight_dtype;
+  float* state;
+  const int* tok_slot;
+  const int* tok_pos;
+  const int* seq_slot;
+  const int* seq_start;
+  int tokens, batch, channels, taps;
+  void* y;  // [tokens, channels]
+  int y_dtype;
+};
+
+__global__ void conv_silu_kernel(ConvArgs a) {
+  const size_t total = (size_t)a.tokens * a.channels;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int token = (int)(i / a.channels), c = (int)(i % a.channels);
+    const int slot = a.tok_slot[token];
+    if (slot < 0) {
+      store_from_f32(a.y, a.y_dtype, i, 0.0f);
+      continue;
+    }
+    const int pos = a.tok_pos[token];
+    float acc = a.bias ? load_as_f32(a.bias, a.weight_dtype, c) : 0.0f;
+    bool in_step = true;  // the rows token, token - 1, ... while they belong to this sequence
+    int behind = 0;       // how many inputs of the state have been used
+    for (int back = 0; back < a.taps; ++back) {
+      if (back > pos) break;  // before the sequence's start: zeros
+      float v;
+      if (in_step && token - back >= 0 && a.tok_slot[token - back] == slot) {
+        v = load_as_f32(a.x, a.x_dtype, (size_t)(token - back) * a.x_stride + c);
+      } else {
+        in_step = false;
+        ++behind;  // the newest input of the state is its last row
+        v = a.state[((size_t)slot * (a.taps - 1) + (a.taps - 1 - behind)) * a.channels + c];
+      }
+      acc = fmaf(load_as_f32(a.weight, a.weight_dtype, (size_t)c * a.taps + (a.taps - 1 - back)), v, acc);
+    }
+    store_from_f32(a.y, a.y_dtype, i, acc / (1.0f + expf(-acc)));
+  }
+}
+
+// after the outputs are taken: the state becomes the last taps - 1 inputs of each sequence (one thread a
+// channel keeps the old ones it still needs in registers)
+__global__ void conv_state_kernel(ConvArgs a) {
+  const int b = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot < 0 || c >= a.channels) return;
+  const int first = a.seq_start[b], count = a.seq_start[b + 1] - first;
+  if (count <= 0) return;
+  const int keep = a.taps - 1;
+  float* state = a.state + (size_t)slot * keep * a.channels + c;
+  float fresh[kMostTaps];
+#pragma unroll
+  for (int j = 0; j < kMostTaps; ++j) {
+    if (j < keep) {
+      const int back = keep - 1 - j;  // new row j holds the input `back` tokens before the run's last
+      fresh[j] = back < count ? load_as_f32(a.x, a.x_dtype, (size_t)(first + count - 1 - back) * a.x_stride + c)
+                              : state[(size_t)(j + count) * a.channels];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kMostTaps; ++j)
+    if (j < keep) state[(size_t)j * a.channels] = fresh[j];
+}
+
+// -----------------------------------------------------------------------------
+// Selective scan.  Per channel c and state n, over a sequence's tokens:
+//   dt = softplus(dt_pre[t, c] + dt_bias[c])
+//   S[c, n] <- exp(dt * A[c, n]) S[c, n] + dt * x[t, c] * B[t, n]
+//   y[t, c] = (sum_n S[c, n] C[t, n] + D[c] x[t, c]) * silu(z[t, c])
+// A thread keeps 8 states of one channel; the lanes of a channel (a power of two, up to 16) sit side by side
+// and add their parts of y by lane exchanges.  bc [tokens, 2 * states]: B then C.  A = -exp(A_log) comes
+// ready-made.  state [slots, channels, states].
+// -----------------------------------------------------------------------------
+struct ScanArgs {
+  const void* x;  // [tokens, channels]
+  int x_dtype;
+  const float* dt_pre;  // [tokens, channels]
+  const float* bc;      // [tokens, 2 * states]
+  const void* z;        // [tokens, z_stride]: the first `channels` columns from the pointer on
+  int z_dtype, z_stride;
+  const float* A;        // [channels, states]
+  const float* D;        // [channels]
+  const float* dt_bias;  // [channels]
+  float* state;
+  const int* seq_slot;
+  const int* seq_start;
+  int channels, states;
+  void* y;  // [tokens, channels]
+  int y_dtype;
+};
+
+template <int LANES>
+__global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
+  const int b = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  if (slot < 0) return;
+  const int first = a.seq_start[b], last = a.seq_start[b + 1];
+  if (last <= first) return;
+  const int part = threadIdx.x % LANES;
+  const int c = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
+  const bool live = c < a.channels;
+  const int cc = live ? c : 0;
+  const int N = a.states;
+  float S[8], A[8];
+  float* state = a.state + ((size_t)slot * a.channels + cc) * N;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int n = part * 8 + j;
+    S[j] = (live && n < N) ? state[n] : 0.0f;
+    A[j] = (live && n < N) ? a.A[(size_t)cc * N + n] : 0.0f;
+  }
+  const float D = a.D[cc], dt_bias = a.dt_bias[cc];
+  for (int t = first; t < last; ++t) {
+    const float x = load_as_f32(a.x, a.x_dtype, (size_t)t * a.channels + cc);
+    const float dt = softplus_f(a.dt_pre[(size_t)t * a.channels + cc] + dt_bias);
+    const float* B = a.bc + (size_t)t * 2 * N;
+    const float* C = B + N;
+    const float dx = dt * x;
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = part * 8 + j;
+      if (n < N) {
+        S[j] = fmaf(expf(dt * A[j]), S[j], dx * B[n]);
+        acc = fmaf(S[j], C[n], acc);
+      }
+    }
+#pragma unroll
+    for (int offset = LANES / 2; offset > 0; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
+    if (part == 0 && live) {
+      const float z = load_as_f32(a.z, a.z_dtype, (size_t)t * a.z_stride + c);
+      store_from_f32(a.y, a.y_dtype, (size_t)t * a.channels + c, (acc + D * x) * (z * sigmoid_f(z)));
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = part * 8 + j;
+      if (n < N) state[n] = S[j];
+    }
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Gated linear attention.  Per head, over a sequence's tokens, with a state S [key channels, value channels]:
+//   alpha = sigmoid(zd)^(1 / tau)            per key channel
+//   S <- diag(alpha) S + k v^T
+//   o = S^T (q * scale)
+// A block takes one head of one sequence and a slab of value columns; a thread keeps 16 key rows of one
+// column, the threads of a column (a power of two, up to 16) sit 64 / GROUPS lanes apart in one wave and add
+// their parts of o by lane exchanges.  Tokens come through LDS a chunk at a time (queries, keys, decays of
+// the head and the slab's values), loaded by the whole block.  o is left raw, in 32-bit.
+// -----------------------------------------------------------------------------
+struct GlaArgs {
+  const void* q;  // row t, head h: q + t * q_stride + h * key_dim  (k alike; v, with value_dim)
+  const void* k;
+  const void* v;
+  int qkv_dtype;
+  int q_stride, k_stride, v_stride;
+  const float* zd;  // [tokens, heads * key_dim]: the decays before the sigmoid
+  float inv_tau, scale;
+  float* state;  // [slots, heads, key_dim, value_dim]
+  const int* seq_slot;
+  const int* seq_start;
+  int heads, key_dim, value_dim;
+  int chunk;   // tokens staged at a time
+  float* out;  // [tokens, heads * value_dim]
+};
+
+template <int GROUPS>
+__global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
+  extern __shared__ float lds[];
+  constexpr int kCols = 4 * (kWave / GROUPS);  // value columns of a block (4 waves)
+  const int b = blockIdx.z, head = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  if (slot < 0) return;
+  const int first = a.seq_start[b], last = a.seq_start[b + 1];
+  if (last <= first) return;
+  const int d = a.key_dim, e = a.value_dim;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int group = lane / (kWave / GROUPS);
+  const int col_in_block = wave * (kWave / GROUPS) + lane % (kWave / GROUPS);
+  const int col = blockIdx.x * kCols + col_in_block;
+  const bool live = col < e;
+  float* qs = lds;                    // [chunk][d]
+  float* ks = qs + a.chunk * d;       // [chunk][d]
+  float* as = ks + a.chunk * d;       // [chunk][d]
+  float* vs = as + a.chunk * d;       // [chunk][kCols]
+  float S[16];
+  float* state = a.state + (((size_t)slot * a.heads + head) * d) * e + (live ? col : 0);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = group * 16 + r;
+    S[r] = (live && row < d) ? state[(size_t)row * e] : 0.0f;
+  }
+  for (int t0 = first; t0 < last; t0 += a.chunk) {
+    const int count = min(a.chunk, last - t0);
+    __syncthreads();  // the chunk before has been read
+    for (int i = threadIdx.x; i < count * d; i += blockDim.x) {
+      const int t = t0 + i / d, ch = i % d;
+      qs[i] = load_as_f32(a.q, a.qkv_dtype, (size_t)t * a.q_stride + head * d + ch) * a.scale;
+      ks[i] = load_as_f32(a.k, a.qkv_dtype, (size_t)t * a.k_stride + head * d + ch);
+      as[i] = expf(log_sigmoid_f(a.zd[((size_t)t * a.heads + head) * d + ch]) * a.inv_tau);
+    }
+    for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
+      const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
+      vs[i] = cl < e ? load_as_f32(a.v, a.qkv_dtype, (size_t)t * a.v_stride + head * e + cl) : 0.0f;
+    }
+    __syncthreads();
+    for (int j = 0; j < count; ++j) {
+      const float v = vs[j * kCols + col_in_block];
+      const float* qj = qs + j * d + group * 16;
+      const float* kj = ks + j * d + group * 16;
+      const float* aj = as + j * d + group * 16;
+      float acc = 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if (group * 16 + r < d) {
+          S[r] = fmaf(aj[r], S[r], kj[r] * v);
+          acc = fmaf(S[r], qj[r], acc);
+        }
+      }
+#pragma unroll
+      for (int offset = kWave / 2; offset >= kWave / GROUPS; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
+      if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = group * 16 + r;
+      if (row < d) state[(size_t)row * e] = S[r];
+    }
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Behind the scan: each head's o normed by its root mean square over its channels, times a weight shared by
+// the heads, times silu(gate):  y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(g[t, h, :]).  A wave a (token, head).
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const void* __restrict__ gate, int gate_dtype,
+                                                             int gate_stride, const void* __restrict__ weight, int weight_dtype,
+                                                             void* __restrict__ y, int y_dtype, int items, int heads, int dim, float eps) {
+  const int item = blockIdx.x * 4 + threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  if (item >= items) return;
+  const int token = item / heads, head = item % heads;
+  const float* row = o + (size_t)item * dim;
+  float squares = 0.0f;
+  for (int c = lane; c < dim; c += kWave) squares = fmaf(row[c], row[c], squares);
+  const float scale = 1.0f / sqrtf(wave_sum(squares) / (float)dim + eps);
+  for (int c = lane; c < dim; c += kWave) {
+    const float g = load_as_f32(gate, gate_dtype, (size_t)token * gate_stride + head * dim + c);
+    const float v = (row[c] * scale) * load_as_f32(weight, weight_dtype, c);
+    store_from_f32(y, y_dtype, (size_t)item * dim + c, v * (g * sigmoid_f(g)));
+  }
+}
+
+}  // namespace
+
+extern "C" int nnis_conv_silu(const void* x, int x_dtype, int x_stride, const void* weight, const void* bias, int weight_dtype,
+                              float* state, const int* tok_slot, const int* tok_pos, const int* seq_slot, const int* seq_start,
+                              int tokens, int batch, int channels, int taps, void* y, int y_dtype, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(y_dtype), "conv: unknown dtype");
+  NNIS_REQUIRE(taps >= 1 && taps <= kMostTaps, "conv: 1 to %d taps are taken, got %d", kMostTaps, taps);
+  NNIS_REQUIRE(channels > 0 && x_stride >= channels && tokens >= 0 && batch >= 0, "conv: bad sizes");
+  NNIS_REQUIRE(x && weight && tok_slot && tok_pos && seq_slot && seq_start && y && (state || taps == 1), "conv: a pointer is missing");
+  if (tokens == 0 || batch == 0) return 0;
+  ConvArgs a;
+  a.x = x; a.x_dtype = x_dtype; a.x_stride = x_stride; a.weight = weight; a.bias = bias; a.weight_dtype = weight_dtype; a.state = state;
+  a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.seq_slot = seq_slot; a.seq_start = seq_start; a.tokens = tokens; a.batch = batch;
+  a.channels = channels; a.taps = taps; a.y = y; a.y_dtype = y_dtype;
+  const size_t total = (size_t)tokens * channels;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("conv_silu");
+  if (taps > 1) {
+    const int threads = channels >= 256 ? 256 : 64;
+    hipLaunchKernelGGL(conv_state_kernel, dim3((channels + threads - 1) / threads, batch), dim3(threads), 0, (hipStream_t)stream, a);
+    NNIS_LAUNCH_CHECK("conv_state");
+  }
+  return 0;
+}
+
+extern "C" int nnis_selective_scan(const void* x, int x_dtype, const float* dt_pre, const float* bc, const void* z, int z_dtype,
+                                   int z_stride, const float* A, const float* D, const float* dt_bias, float* state,
+                                   const int* seq_slot, const int* seq_start, int batch, int channels, int states, void* y,
+                                   int y_dtype, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(z_dtype) && nnis_dtype_ok(y_dtype), "selective_scan: unknown dtype");
+  NNIS_REQUIRE(channels > 0 && states > 0 && states <= 128 && z_stride >= channels && batch >= 0,
+               "selective_scan: bad sizes (channels %d, states %d: up to 128 are taken)", channels, states);
+  NNIS_REQUIRE(x && dt_pre && bc && z && A && D && dt_bias && state && seq_slot && seq_start && y, "selective_scan: a pointer is missing");
+  if (batch == 0) return 0;
+  ScanArgs a;
+  a.x = x; a.x_dtype = x_dtype; a.dt_pre = dt_pre; a.bc = bc; a.z = z; a.z_dtype = z_dtype; a.z_stride = z_stride; a.A = A; a.D = D;
+  a.dt_bias = dt_bias; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.channels = channels; a.states = states;
+  a.y = y; a.y_dtype = y_dtype;
+  const int need = (states + 7) / 8;
+  hipStream_t s = (hipStream_t)stream;
+#define NNIS_SCAN(LANES_)                                                                                                  \
+  hipLaunchKernelGGL(selective_scan_kernel<LANES_>, dim3((channels + 256 / LANES_ - 1) / (256 / LANES_), batch), dim3(256), 0, s, a)
+  if (need <= 1) NNIS_SCAN(1);
+  else if (need <= 2) NNIS_SCAN(2);
+  else if (need <= 4) NNIS_SCAN(4);
+  else if (need <= 8) NNIS_SCAN(8);
+  else NNIS_SCAN(16);
+#undef NNIS_SCAN
+  NNIS_LAUNCH_CHECK("selective_scan");
+  return 0;
+}
+
+extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
+                             const float* zd, float tau, float scale, float* state, const int* seq_slot, const int* seq_start,
+                             int batch, int heads, int key_dim, int value_dim, float* out, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype), "gla_scan: unknown dtype %d", qkv_dtype);
+  NNIS_REQUIRE(heads > 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
+               "gla_scan: bad sizes (heads %d, key channels %d: up to 256 are taken, value channels %d)", heads, key_dim, value_dim);
+  NNIS_REQUIRE(tau > 0.0f, "gla_scan: tau must be positive, got %g", (double)tau);
+  NNIS_REQUIRE(q && k && v && zd && state && seq_slot && seq_start && out, "gla_scan: a pointer is missing");
+  if (batch == 0) return 0;
+  GlaArgs a;
+  a.q = q; a.k = k; a.v = v; a.qkv_dtype = qkv_dtype; a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.zd = zd;
+  a.inv_tau = 1.0f / tau; a.scale = scale; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads;
+  a.key_dim = key_dim; a.value_dim = value_dim; a.out = out;
+  const int need = (key_dim + 15) / 16;
+  const int groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
+  const int cols = 4 * (kWave / groups);
+  int chunk = (int)((40 * 1024) / ((3 * (size_t)key_dim + cols) * sizeof(float)));
+  chunk = chunk > 32 ? 32 : (chunk < 1 ? 1 : chunk);
+  a.chunk = chunk;
+  const size_t lds = (size_t)chunk * (3 * key_dim + cols) * sizeof(float);
+  const dim3 grid((value_dim + cols - 1) / cols, heads, batch);
+  hipStream_t s = (hipStream_t)stream;
+  switch (groups) {
+    case 1: hipLaunchKernelGGL(gla_scan_kernel<1>, grid, dim3(256), lds, s, a); break;
+    case 2: hipLaunchKernelGGL(gla_scan_kernel<2>, grid, dim3(256), lds, s, a); break;
+    case 4: hipLaunchKernelGGL(gla_scan_kernel<4>, grid, dim3(256), lds, s, a); break;
+    case 8: hipLaunchKernelGGL(gla_scan_kernel<8>, grid, dim3(256), lds, s, a); break;
+    default: hipLaunchKernelGGL(gla_scan_kernel<16>, grid, dim3(256), lds, s, a); break;
+  }
+  NNIS_LAUNCH_CHECK("gla_scan");
+  return 0;
+}
+
+extern "C" int nnis_head_norm_gate(const float* o, const void* gate, int gate_dtype, int gate_stride, const void* weight,
+                                   int weight_dtype, void* y, int y_dtype, int tokens, int heads, int dim, float eps, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(gate_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(y_dtype), "head_norm_gate: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && heads > 0 && dim > 0 && gate_stride >= heads * dim && eps > 0.0f, "head_norm_gate: bad sizes");
+  NNIS_REQUIRE(o && gate && weight && y, "head_norm_gate: a pointer is missing");
+  const int items = tokens * heads;
+  if (items == 0) return 0;
+  hipLaunchKernelGGL(head_norm_gate_kernel, dim3((items + 3) / 4), dim3(256), 0, (hipStream_t)stream, o, gate, gate_dtype, gate_stride,
+                     weight, weight_dtype, y, y_dtype, items, heads, dim, eps);
+  NNIS_LAUNCH_CHECK("head_norm_gate");
+  return 0;
+}

@@ -1,0 +1,309 @@
+// Row-wise kernels around a residual that is kept as several streams, and the small fused steps of mixers
+// that run side by side: an embedding with a hashed table of token pairs, the streams' update and weighted
+// sum fused with the norm that follows, the mean of branches each normed by its root mean square, a gated
+// activation with a choice of activation, and a bias added in place.
+// Storage types are chosen at run time; every sum and statistic is 32-bit.
+#include "common.h"
+
+// -----------------------------------------------------------------------------
+// Embedding with a table of token pairs: out[c][t, :] = table[id] + pairs[row], the same in every one of
+// `copies` copies.  row = (previous * mul_prev + id * mul_cur) % buckets, or `buckets` (the table's last
+// row) for a sequence's first token.  The token before the first one a step brings for a sequence is kept
+// per slot in `last_token`; the block of a run's first row reads it and then stores the run's last id
+// there (no other block reads that word).  Rows of one sequence follow one another and a slot appears in
+// one run only.  A padding row (negative slot or id outside the table) is zero.
+// -----------------------------------------------------------------------------
+__global__ void embed_pair_kernel(const int* __restrict__ ids, const int* __restrict__ tok_slot, const int* __restrict__ tok_pos,
+                                  int tokens, const void* __restrict__ table, int table_dtype, int vocab,
+                                  const void* __restrict__ pairs, int pairs_dtype, int buckets, long long mul_prev,
+                                  long long mul_cur, int* __restrict__ last_token, float* __restrict__ out, int copies, int width) {
+  __shared__ int s_before;
+  const int token = blockIdx.x;
+  const int id = ids[token];
+  const int slot = tok_slot[token];
+  const size_t plane = (size_t)tokens * width;
+  float* dst = out + (size_t)token * width;
+  if (slot < 0 || id < 0 || id >= vocab) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x)
+      for (int s = 0; s < copies; ++s) dst[s * plane + c] = 0.0f;
+    return;
+  }
+  const int pos = tok_pos[token];
+  const bool starts_run = token == 0 || tok_slot[token - 1] != slot;
+  if (threadIdx.x == 0) s_before = starts_run ? last_token[slot] : ids[token - 1];
+  __syncthreads();
+  const int before = s_before;
+  if (starts_run) {
+    // the last row of this run leaves its id for the step that comes next
+    for (int r = token + threadIdx.x; r < tokens && tok_slot[r] == slot; r += blockDim.x)
+      if (r + 1 == tokens || tok_slot[r + 1] != slot) last_token[slot] = ids[r];
+  }
+  long long row = buckets;
+  if (pos > 0 && before >= 0) row = ((long long)before * mul_prev + (long long)id * mul_cur) % buckets;
+  const size_t base = (size_t)id * width, pair_base = (size_t)row * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = load_as_f32(table, table_dtype, base + c) + load_as_f32(pairs, pairs_dtype, pair_base + c);
+    for (int s = 0; s < copies; ++s) dst[s * plane + c] = v;
+  }
+}
+
+extern "C" int nnis_embed_pair(const int* ids, const int* tok_slot, const int* tok_pos, int tokens, const void* table,
+                               int table_dtype, int vocab, const void* pairs, int pairs_dtype, int buckets, long long mul_prev,
+                               long long mul_cur, int* last_token, float* out, int copies, int width, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(table_dtype) && nnis_dtype_ok(pairs_dtype), "embed_pair: unknown table dtype");
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0 && buckets > 0 && copies > 0, "embed_pair: bad sizes");
+  NNIS_REQUIRE(mul_prev >= 0 && mul_cur >= 0, "embed_pair: the multipliers must not be negative");
+  NNIS_REQUIRE(ids && tok_slot && tok_pos && last_token && out, "embed_pair: a pointer is missing");
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(embed_pair_kernel, dim3(tokens), dim3(width >= 1024 ? 256 : 64), 0, (hipStream_t)stream, ids, tok_slot,
+                     tok_pos, tokens, table, table_dtype, vocab, pairs, pairs_dtype, buckets, mul_prev, mul_cur, last_token, out,
+                     copies, width);
+  NNIS_LAUNCH_CHECK("embed_pair");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Streams.  x [streams, tokens, width] in 32-bit.  One block a row, in up to three steps:
+//   update (y given):  x_t <- sum_s mix[s, t] x_s + gain[t] * y      all streams at once, in place
+//   read:              u = sum_t take[t] x_t                         (take null: every stream counts once)
+//   norm (weight given): h = (u - mean) / sqrt(var + eps) * weight + bias, var the mean squared deviation
+//                        (centred = 0: h = u / sqrt(mean(u^2) + eps) * weight [+ bias])
+// Without a norm weight, h = u.  With `rows`, output row r reads input row rows[r] (then nothing is updated).
+// u is held in LDS between the passes (width floats).
+// -----------------------------------------------------------------------------
+constexpr int kMostStreams = 8;
+
+struct StreamArgs {
+  float* x;
+  int streams, tokens, width;
+  const void* y;  // [tokens, width] or null
+  int y_dtype;
+  const float* mix;   // [streams, streams], [from, to]
+  const float* gain;  // [streams]
+  const float* take;  // [streams] or null
+  const void* weight;  // [width] or null
+  const void* bias;    // [width] or null
+  int weight_dtype;
+  int centred;
+  float eps;
+  void* h;  // [out_rows, width] or null
+  int h_dtype;
+  const int* rows;
+};
+
+__global__ void stream_kernel(StreamArgs a) {
+  extern __shared__ float u_row[];
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int row = a.rows ? a.rows[out_row] : out_row;
+  const int S = a.streams;
+  const size_t plane = (size_t)a.tokens * a.width;
+  float* x = a.x + (size_t)row * a.width;
+  float mix[kMostStreams][kMostStreams], gain[kMostStreams], take[kMostStreams];
+#pragma unroll
+  for (int s = 0; s < kMostStreams; ++s) {
+    take[s] = s < S ? (a.take ? a.take[s] : 1.0f) : 0.0f;
+    gain[s] = (a.y && s < S) ? a.gain[s] : 0.0f;
+#pragma unroll
+    for (int t = 0; t < kMostStreams; ++t) mix[s][t] = (a.y && s < S && t < S) ? a.mix[s * S + t] : 0.0f;
+  }
+  float sum = 0.0f;
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    float v[kMostStreams];
+#pragma unroll
+    for (int s = 0; s < kMostStreams; ++s) v[s] = s < S ? x[s * plane + c] : 0.0f;
+    if (a.y) {
+      const float y = load_as_f32(a.y, a.y_dtype, (size_t)row * a.width + c);
+      float w[kMostStreams];
+#pragma unroll
+      for (int t = 0; t < kMostStreams; ++t) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < kMostStreams; ++s) acc = fmaf(mix[s][t], v[s], acc);
+        w[t] = fmaf(gain[t], y, acc);
+      }
+#pragma unroll
+      for (int t = 0; t < kMostStreams; ++t) {
+        v[t] = w[t];
+        if (t < S) x[t * plane + c] = w[t];
+      }
+    }
+    float u = 0.0f;
+#pragma unroll
+    for (int s = 0; s < kMostStreams; ++s) u = fmaf(take[s], v[s], u);
+    u_row[c] = u;
+    sum += u;
+  }
+  if (a.h == nullptr) return;
+  const size_t out_base = (size_t)out_row * a.width;
+  if (a.weight == nullptr) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < a.width; c += blockDim.x) store_from_f32(a.h, a.h_dtype, out_base + c, u_row[c]);
+    return;
+  }
+  const float inv_width = 1.0f / (float)a.width;
+  const float mean = a.centred ? block_sum(sum, scratch) * inv_width : 0.0f;  // (block_sum's barriers order the LDS writes)
+  float squares = 0.0f;
+  if (!a.centred) __syncthreads();
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    const float d = u_row[c] - mean;
+    squares = fmaf(d, d, squares);
+  }
+  const float scale = 1.0f / sqrtf(block_sum(squares, scratch) * inv_width + a.eps);
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    float v = ((u_row[c] - mean) * scale) * load_as_f32(a.weight, a.weight_dtype, c);
+    if (a.bias) v += load_as_f32(a.bias, a.weight_dtype, c);
+    store_from_f32(a.h, a.h_dtype, out_base + c, v);
+  }
+}
+
+extern "C" int nnis_stream_step(float* x, int streams, int tokens, int width, const void* y, int y_dtype, const float* mix,
+                                const float* gain, const float* take, const void* weight, const void* bias, int weight_dtype,
+                                int centred, float eps, void* h, int h_dtype, const int* rows, int out_rows, void* stream) {
+  NNIS_REQUIRE(streams >= 1 && streams <= kMostStreams, "streams: 1 to %d streams are taken, got %d", kMostStreams, streams);
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && width <= 16384, "streams: bad sizes tokens=%d width=%d", tokens, width);
+  NNIS_REQUIRE(x != nullptr, "streams: x is missing");
+  NNIS_REQUIRE(y == nullptr || (nnis_dtype_ok(y_dtype) && mix && gain && rows == nullptr),
+               "streams: an update needs mix and gain and no row list");
+  NNIS_REQUIRE(h == nullptr || nnis_dtype_ok(h_dtype), "streams: unknown output dtype %d", h_dtype);
+  NNIS_REQUIRE(weight == nullptr || (nnis_dtype_ok(weight_dtype) && eps > 0.0f && h != nullptr), "streams: a norm needs a weight type, eps and an output");
+  NNIS_REQUIRE(bias == nullptr || weight != nullptr, "streams: a bias comes with a weight");
+  NNIS_REQUIRE(h != nullptr || y != nullptr, "streams: nothing to do");
+  if (out_rows <= 0) return 0;
+  StreamArgs a;
+  a.x = x; a.streams = streams; a.tokens = tokens; a.width = width; a.y = y; a.y_dtype = y_dtype; a.mix = mix; a.gain = gain;
+  a.take = take; a.weight = weight; a.bias = bias; a.weight_dtype = weight_dtype; a.centred = centred; a.eps = eps; a.h = h;
+  a.h_dtype = h_dtype; a.rows = rows;
+  const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  hipLaunchKernelGGL(stream_kernel, dim3(out_rows), dim3(threads), (size_t)width * sizeof(float), (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("stream_step");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Branches side by side: out = (1 / n) sum_i  (y_i + b_i) / sqrt(mean((y_i + b_i)^2) + eps) * w_i,
+// the mean over the row.  Up to kMostBranches inputs [tokens, width], each with a weight and, optionally, a
+// bias that its producer has not added yet.  One block a row.
+// -----------------------------------------------------------------------------
+constexpr int kMostBranches = 4;
+
+struct BranchArgs {
+  const void* y[kMostBranches];
+  const void* weight[kMostBranches];
+  const void* bias[kMostBranches];
+  int count;
+  int y_dtype, weight_dtype;
+  int width;
+  float eps;
+  void* out;
+  int out_dtype;
+};
+
+__global__ void branch_mean_kernel(BranchArgs a) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * a.width;
+  float scale[kMostBranches];
+#pragma unroll
+  for (int i = 0; i < kMostBranches; ++i) {
+    scale[i] = 0.0f;
+    if (i < a.count) {
+      float squares = 0.0f;
+      for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+        float v = load_as_f32(a.y[i], a.y_dtype, base + c);
+        if (a.bias[i]) v += load_as_f32(a.bias[i], a.weight_dtype, c);
+        squares = fmaf(v, v, squares);
+      }
+      scale[i] = 1.0f / sqrtf(block_sum(squares, scratch) / (float)a.width + a.eps);
+    }
+  }
+  const float share = 1.0f / (float)a.count;
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kMostBranches; ++i)
+      if (i < a.count) {
+        float v = load_as_f32(a.y[i], a.y_dtype, base + c);
+        if (a.bias[i]) v += load_as_f32(a.bias[i], a.weight_dtype, c);
+        acc += (v * scale[i]) * load_as_f32(a.weight[i], a.weight_dtype, c);
+      }
+    store_from_f32(a.out, a.out_dtype, base + c, acc * share);
+  }
+}
+
+extern "C" int nnis_branch_mean(const void* const* y, const void* const* weight, const void* const* bias, int count, int y_dtype,
+                                int weight_dtype, int tokens, int width, float eps, void* out, int out_dtype, void* stream) {
+  NNIS_REQUIRE(count >= 1 && count <= kMostBranches, "branch_mean: 1 to %d branches are taken, got %d", kMostBranches, count);
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(out_dtype), "branch_mean: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && eps > 0.0f, "branch_mean: bad sizes tokens=%d width=%d", tokens, width);
+  if (tokens == 0) return 0;
+  BranchArgs a;
+  for (int i = 0; i < kMostBranches; ++i) {
+    a.y[i] = i < count ? y[i] : nullptr;
+    a.weight[i] = i < count ? weight[i] : nullptr;
+    a.bias[i] = i < count ? bias[i] : nullptr;
+    NNIS_REQUIRE(i >= count || (a.y[i] && a.weight[i]), "branch_mean: branch %d has no input or no weight", i);
+  }
+  a.count = count; a.y_dtype = y_dtype; a.weight_dtype = weight_dtype; a.width = width; a.eps = eps; a.out = out; a.out_dtype = out_dtype;
+  const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  hipLaunchKernelGGL(branch_mean_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("branch_mean");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Gated activation on a fused [tokens, 2 * inner] projection (gate columns first): out = act(gate) * up.
+//   act 0: SiLU, gate / (1 + exp(-gate))
+//   act 1: the tanh form of GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
+// -----------------------------------------------------------------------------
+__device__ __forceinline__ float gate_activation(float g, int act) {
+  if (act == 0) return g / (1.0f + expf(-g));
+  const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+  return 0.5f * g * (1.0f + tanhf(inner));
+}
+
+__global__ void gated_act_kernel(const void* __restrict__ gate_up, int in_dtype, void* __restrict__ out, int out_dtype, int inner,
+                                 size_t total, int act) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t row = i / inner, col = i % inner;
+    const float g = load_as_f32(gate_up, in_dtype, row * 2 * inner + col);
+    const float u = load_as_f32(gate_up, in_dtype, row * 2 * inner + inner + col);
+    store_from_f32(out, out_dtype, i, gate_activation(g, act) * u);
+  }
+}
+
+extern "C" int nnis_gated_act(const void* gate_up, int in_dtype, void* out, int out_dtype, int tokens, int inner, int act,
+                              void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(in_dtype) && nnis_dtype_ok(out_dtype), "gated_act: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && inner > 0, "gated_act: bad sizes tokens=%d inner=%d", tokens, inner);
+  NNIS_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation %d", act);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * inner;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(gated_act_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, gate_up, in_dtype, out,
+                     out_dtype, inner, total, act);
+  NNIS_LAUNCH_CHECK("gated_act");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// y[t, c] += bias[c], in place
+// -----------------------------------------------------------------------------
+__global__ void add_bias_kernel(void* __restrict__ y, int y_dtype, const void* __restrict__ bias, int bias_dtype, int width,
+                                size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    store_from_f32(y, y_dtype, i, load_as_f32(y, y_dtype, i) + load_as_f32(bias, bias_dtype, i % width));
+}
+
+extern "C" int nnis_add_bias(void* y, int y_dtype, const void* bias, int bias_dtype, int tokens, int width, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(bias_dtype), "add_bias: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && y && bias, "add_bias: bad arguments");
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * width;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(add_bias_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, y, y_dtype, bias, bias_dtype, width,
+                     total);
+  NNIS_LAUNCH_CHECK("add_bias");
+  return 0;
+}

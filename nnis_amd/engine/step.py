@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from ..cache import SequenceCache
+from ..cache.allocator import PAGE_TOKENS, pages_for
 from ..errors import InvalidInput
 from .batch import StepContext, StepEntry
 from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs, prompt_rows
@@ -28,9 +29,10 @@ class Engine:
         self.rt = rt
         model.check(rt)  # (a model that was not loaded through ``load_model``: sizes the kernels refuse stop here)
         self.vocab_size = model.spec.vocab_size
-        self.max_positions = model.spec.max_positions
+        # a model that names no last position can go as far as the cache holds a single sequence
+        self.max_positions = model.spec.max_positions or pages_for(max_tokens) * PAGE_TOKENS
         requests, shared = model.cache_requests()
-        self.cache = SequenceCache(requests, shared, max_tokens, model.spec.max_positions, rt.dtype, rt.device, max_slots)
+        self.cache = SequenceCache(requests, shared, max_tokens, self.max_positions, rt.dtype, rt.device, max_slots)
         self._staging = None
         self._staging_dev = None
         self._staged = None  # recorded behind the staging copy
@@ -43,6 +45,7 @@ class Engine:
         # A step's positions index the rotation tables on the device, where nothing can refuse them: the tables
         # reach as far as the cache lets a sequence grow, so the check of the lengths before a step covers both.
         for name, position in model.positions.items():
+            position.reach(self.max_positions)
             tables = position.rotary()
             if tables is not None and tables.cos.shape[0] < self.max_positions:
                 raise InvalidInput(f"position encoding {name!r} has tables for {tables.cos.shape[0]} positions; "

@@ -49,6 +49,7 @@ FLAGS = [
 # in scratch memory, all outside their loops over the keys; no other kernel of either file spills.)
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
+PREBUILT_WIDE_VALUES = ("attn_hd32v64", "attn_hd64v128", "attn_hd16v48")  # values of another size than the keys: what the tests use
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -98,17 +99,25 @@ def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], r
 
 
 def _attention_recipe(rest: str) -> ModuleRecipe:
+    """``attn_hd<N>``: keys and values of N channels; ``attn_hd<N>v<M>``: values of M."""
     try:
-        head_dim = int(rest)
+        sizes = [int(part) for part in rest.split("v")]
+        if not 1 <= len(sizes) <= 2 or min(sizes) <= 0:
+            raise ValueError(rest)
     except ValueError:
         raise KernelError(f"unknown kernel module 'attn_hd{rest}'") from None
-    return ModuleRecipe(("attention.hip",), ("common.h",), (("NNIS_HEAD_DIM", str(head_dim)),), (("attention.hip", tuple(_VECTOR_SUMS)),))
+    defines = [("NNIS_HEAD_DIM", str(sizes[0]))]
+    if len(sizes) == 2:
+        defines.append(("NNIS_VALUE_DIM", str(sizes[1])))
+    return ModuleRecipe(("attention.hip",), ("common.h",), tuple(defines), (("attention.hip", tuple(_VECTOR_SUMS)),))
 
 
 # the library's own modules: ``core`` holds the kernels whose sizes are run-time arguments; attention is compiled per head size
-register_module("core", ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"],
+register_module("core", ["elementwise.hip", "residual.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"],
                 headers=["common.h", "epilogue.h", "nnis_noalloc.h"], source_flags={"gemm_mfma.hip": _VECTOR_SUMS})
 register_module_family("attn_hd", _attention_recipe)
+# the mixers that carry a state of fixed size (convolution, selective scan, gated linear attention)
+register_module("recurrent", ["recurrent.hip"], headers=["common.h"])
 # plain host references of the kernels' operations, for the tests (no device code: the host compiler builds them)
 register_module("reference", ["reference.cpp"], host_only=True)
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off"]  # a multiply-add is fused only where the source says fmaf
@@ -282,7 +291,7 @@ def load_module(module: str, build_if_missing: bool = True) -> ctypes.CDLL:
 
 
 def all_prebuilt_modules() -> List[str]:
-    return ["core", "reference"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS]
+    return ["core", "reference", "recurrent"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS] + list(PREBUILT_WIDE_VALUES)
 
 
 def build_all(force: bool = True, jobs: int = 4) -> List[str]:

@@ -21,6 +21,7 @@ _INT = ctypes.c_int
 _FLT = ctypes.c_float
 _SIZE = ctypes.c_size_t
 _U64 = ctypes.c_uint64
+_I64 = ctypes.c_longlong
 
 _CORE_SIGNATURES = {
     "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
@@ -29,7 +30,15 @@ _CORE_SIGNATURES = {
     "nnis_rmsnorm": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
                            _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_rope_kv_write_wide": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
+                                _VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID],
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_embed_pair": [_VOID, _VOID, _VOID, _INT, _VOID, _INT, _INT, _VOID, _INT, _INT, _I64, _I64, _VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_stream_step": [_VOID, _INT, _INT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _FLT, _VOID, _INT,
+                         _VOID, _INT, _VOID],
+    "nnis_branch_mean": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT, _VOID, _INT, _VOID],
+    "nnis_gated_act": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_add_bias": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID, _VOID],
     "nnis_argmax_scratch": [_INT, _INT],
     "nnis_argmax_static": [_VOID, _VOID, _INT, _INT, _VOID],
@@ -51,7 +60,7 @@ _CORE_SIGNATURES = {
 }
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
-                            _INT, _INT, _FLT, _VOID],
+                            _INT, _INT, _FLT, _INT, _FLT, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
@@ -62,12 +71,23 @@ _ATTN_SIGNATURES = {
     "nnis_attention_decode_max_waves": [_INT, _INT],
 }
 
+_RECURRENT_SIGNATURES = {
+    "nnis_conv_silu": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT,
+                       _VOID],
+    "nnis_selective_scan": [_VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT,
+                            _VOID, _INT, _VOID],
+    "nnis_gla_scan": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT,
+                      _VOID, _VOID],
+    "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
+}
+
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
 
-def _pages_fit(k_pages: torch.Tensor, v_pages: torch.Tensor, kv_heads: int, head_dim: int) -> bool:
+def _pages_fit(k_pages: torch.Tensor, v_pages: torch.Tensor, kv_heads: int, head_dim: int, value_dim: Optional[int] = None) -> bool:
     """Key and value pages [pages, ...] in the cache's layout for these sizes, contiguous."""
-    return (tuple(k_pages.shape[1:]) == k_page_shape(kv_heads, head_dim) and tuple(v_pages.shape[1:]) == v_page_shape(kv_heads, head_dim)
+    return (tuple(k_pages.shape[1:]) == k_page_shape(kv_heads, head_dim)
+            and tuple(v_pages.shape[1:]) == v_page_shape(kv_heads, value_dim or head_dim)
             and k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.shape[0] == v_pages.shape[0])
 
 
@@ -109,6 +129,15 @@ def _bind(module: str, signatures):
 
 _core = None
 _attn = {}
+_recurrent = None
+
+
+def recurrent():
+    """The module of the mixers that carry state (convolution, selective scan, gated linear attention)."""
+    global _recurrent
+    if _recurrent is None:
+        _recurrent = _bind("recurrent", _RECURRENT_SIGNATURES)
+    return _recurrent
 
 
 def core():
@@ -121,17 +150,26 @@ def core():
 ATTENTION_MOST_CHANNELS = 256
 
 
-def attention_check(head_dim: int) -> None:
+def attention_check(head_dim: int, value_dim: Optional[int] = None) -> None:
     """Raises ``Unsupported`` for a head size that no attention kernel here takes."""
     if head_dim <= 0 or head_dim % 2 != 0 or head_dim > ATTENTION_MOST_CHANNELS:
         raise Unsupported(f"the attention kernels take an even head_dim up to {ATTENTION_MOST_CHANNELS}, got {head_dim}")
+    if value_dim is not None and value_dim != head_dim and not 0 < value_dim <= ATTENTION_MOST_CHANNELS:
+        raise Unsupported(f"the attention kernels take values of up to {ATTENTION_MOST_CHANNELS} channels, got {value_dim}")
 
 
-def attention_module(head_dim: int):
-    if head_dim not in _attn:
-        attention_check(head_dim)
-        _attn[head_dim] = _bind(f"attn_hd{head_dim}", _ATTN_SIGNATURES)
-    return _attn[head_dim]
+def attention_module_name(head_dim: int, value_dim: Optional[int] = None) -> str:
+    """The module compiled for keys of ``head_dim`` channels and values of ``value_dim`` (None: as the keys)."""
+    wide = value_dim is not None and value_dim != head_dim
+    return f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}"
+
+
+def attention_module(head_dim: int, value_dim: Optional[int] = None):
+    name = attention_module_name(head_dim, value_dim)
+    if name not in _attn:
+        attention_check(head_dim, value_dim)
+        _attn[name] = _bind(name, _ATTN_SIGNATURES)
+    return _attn[name]
 
 
 def _check(lib, status: int) -> None:
@@ -233,17 +271,24 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                   rot_dim: int, tok_slot: torch.Tensor, tok_pos: torch.Tensor, k_pages: Optional[torch.Tensor],
                   v_pages: Optional[torch.Tensor], block_table: Optional[torch.Tensor], heads: int, kv_heads: int,
-                  head_dim: int) -> torch.Tensor:
+                  head_dim: int, value_dim: Optional[int] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotates queries and keys by their positions and writes keys and values
     into the pages of each token's slot.  ``k_pages`` and ``v_pages`` are
     ``[pages, *k_page_shape(kv_heads, head_dim)]`` and ``[pages,
-    *v_page_shape(kv_heads, head_dim)]`` (``cache/layout.py``); both ``None``
-    for a run that keeps no cache of its own."""
+    *v_page_shape(kv_heads, value_dim)]`` (``cache/layout.py``); both ``None``
+    for a run that keeps no cache of its own.  ``value_dim``: channels of a
+    value head (None: as the keys).  ``bias``: one entry per column of
+    ``qkv``, added before the rotation."""
     _dev(qkv, "qkv"), _dev(q_out, "q_out"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
     tokens = qkv.shape[0]
-    if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim or q_out.shape != (tokens, heads * head_dim):
+    value_dim = value_dim or head_dim
+    if qkv.shape[1] != (heads + kv_heads) * head_dim + kv_heads * value_dim or q_out.shape != (tokens, heads * head_dim):
         raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} / q_out {tuple(q_out.shape)} do not fit "
-                          f"{heads}+2*{kv_heads} heads of {head_dim}")
+                          f"{heads}+{kv_heads} heads of {head_dim} and {kv_heads} of {value_dim}")
+    if bias is not None:
+        _dev(bias, "bias")
+        if bias.numel() != qkv.shape[1]:
+            raise KernelError(f"rope_kv_write: a bias of {bias.numel()} entries for rows of {qkv.shape[1]}")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or tok_slot.numel() < tokens or tok_pos.numel() < tokens:
         raise KernelError("rope_kv_write: tok_slot / tok_pos must be int32 with one entry per token")
     table_positions = 0
@@ -256,17 +301,18 @@ def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Te
     cache_code = 0
     if k_pages is not None:
         _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
-        if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
+        if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
             raise KernelError(f"rope_kv_write: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
         if block_table.dtype != torch.int32 or block_table.dim() != 2:
             raise KernelError("rope_kv_write: block_table must be int32 [slots, pages]")
         max_pages = block_table.shape[1]
         cache_code = _code(k_pages)
     lib = core()
-    _check(lib, lib.nnis_rope_kv_write(qkv.data_ptr(), _code(qkv), q_out.data_ptr(), _code(q_out), _ptr(cos), _ptr(sin),
-                                       table_positions, rot_dim, tok_slot.data_ptr(), tok_pos.data_ptr(),
-                                       _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, tokens,
-                                       heads, kv_heads, head_dim, _stream()))
+    _check(lib, lib.nnis_rope_kv_write_wide(qkv.data_ptr(), _code(qkv), q_out.data_ptr(), _code(q_out), _ptr(cos), _ptr(sin),
+                                            table_positions, rot_dim, tok_slot.data_ptr(), tok_pos.data_ptr(),
+                                            _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, tokens,
+                                            heads, kv_heads, head_dim, value_dim, _ptr(bias),
+                                            _code(bias) if bias is not None else 0, _stream()))
     return q_out
 
 
@@ -384,24 +430,29 @@ def step_tables(tok_slot: torch.Tensor, tok_pos: torch.Tensor, tokens: int, cos:
 
 def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                    block_table: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, heads: int, kv_heads: int,
-                   head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+                   head_dim: int, scale: float, window: int = 0, value_dim: Optional[int] = None,
+                   softcap: float = 0.0) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its slot up to
-    its own position (32-bit arithmetic, any storage type)."""
+    its own position (32-bit arithmetic, any storage type).  ``value_dim``:
+    channels of a value head and of a head's output (None: as the keys).
+    ``softcap`` > 0: a score s counts as softcap * tanh(s / softcap)."""
     _dev(q, "q"), _dev(out, "out"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
     tokens = q.shape[0]
-    if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
-        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
-    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
+    value_dim = value_dim or head_dim
+    if q.shape != (tokens, heads * head_dim) or out.shape != (tokens, heads * value_dim):
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim} "
+                          f"with values of {value_dim}")
+    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
         raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
     if k_pages.dtype != v_pages.dtype:
         raise KernelError("attention: key and value pages differ in type")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
-    lib = attention_module(head_dim)
+    lib = attention_module(head_dim, value_dim)
     _check(lib, lib.nnis_attention_rows(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
                                         v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
                                         tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
-                                        int(window), float(scale), _stream()))
+                                        int(window), float(scale), int(value_dim), float(softcap), _stream()))
     return out
 
 
@@ -986,7 +1037,8 @@ def prefill_tile_list(new_tokens, first_positions, padded, rows: int):
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
-              window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None, plan=None):
+              window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None, plan=None,
+              value_dim: Optional[int] = None, softcap: float = 0.0):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
     tokens, one for runs of tokens); anything else takes the 32-bit kernel.
@@ -995,7 +1047,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     ``plan``: (runs, waves) of a step of single tokens (``decode_plan``), or
     (waves, columns) of a step of prompts (``prefill_plan``); None: as those
     functions choose for the step's planned sizes."""
-    fast = (q.dtype == torch.bfloat16 and view.k_pages.dtype == torch.bfloat16 and head_dim % 16 == 0)
+    value_dim = value_dim or head_dim
+    fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap)
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
         splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * head_dim)
         waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
@@ -1017,7 +1070,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
                                       waves, columns)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
-                          kv_heads, head_dim, scale, window)
+                          kv_heads, head_dim, scale, window, value_dim, softcap)
+
+
+def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0) -> bool:
+    """Whether ``attention`` takes the matrix-core kernels for these types and sizes (else the 32-bit row kernel)."""
+    return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
+            and (value_dim or head_dim) == head_dim and not softcap)
 
 
 def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, rng: torch.Tensor,
@@ -1056,4 +1115,239 @@ def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, 
     _check(lib, lib.nnis_sample(logits.data_ptr(), weights.data_ptr(), rows, vocab, row_slot.data_ptr(), rng.data_ptr(),
                                 temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), 1 if by_slot else 0,
                                 best.data_ptr(), out.data_ptr(), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# a residual kept as several streams; branches side by side; activations
+# ---------------------------------------------------------------------------
+
+def embed_pair(ids: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor,
+               mul_prev: int, mul_cur: int, last_token: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[c, t, :] = table[ids[t]] + pairs[row] for every copy c of ``out`` [copies, tokens, width] (32-bit), with
+    row = (token before * mul_prev + ids[t] * mul_cur) % (rows of ``pairs`` - 1), or the last row of ``pairs`` for a
+    sequence's first token.  ``last_token`` (int32 [slots]) holds, per slot, the last token of the step before, and
+    is left holding this step's.  Padding rows (negative slot, id outside the table) are zero."""
+    for t, what in ((ids, "ids"), (tok_slot, "tok_slot"), (tok_pos, "tok_pos"), (table, "table"), (pairs, "pairs"),
+                    (last_token, "last_token"), (out, "out")):
+        _dev(t, what)
+    copies, tokens, width = out.shape
+    if out.dtype != torch.float32 or table.dim() != 2 or pairs.dim() != 2 or table.shape[1] != width or pairs.shape[1] != width:
+        raise KernelError(f"embed_pair: tables {tuple(table.shape)} / {tuple(pairs.shape)} do not fit out {tuple(out.shape)} {out.dtype}")
+    if pairs.shape[0] < 2:
+        raise KernelError("embed_pair: the table of pairs needs at least one bucket and the row of a first token")
+    for t in (ids, tok_slot, tok_pos):
+        if t.dtype != torch.int32 or t.numel() < tokens:
+            raise KernelError("embed_pair: ids, tok_slot and tok_pos must be int32 with one entry per token")
+    if last_token.dtype != torch.int32:
+        raise KernelError("embed_pair: last_token must be int32 [slots]")
+    lib = core()
+    _check(lib, lib.nnis_embed_pair(ids.data_ptr(), tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, table.data_ptr(), _code(table),
+                                    table.shape[0], pairs.data_ptr(), _code(pairs), pairs.shape[0] - 1, int(mul_prev), int(mul_cur),
+                                    last_token.data_ptr(), out.data_ptr(), copies, width, _stream()))
+    return out
+
+
+def stream_step(x: torch.Tensor, h: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None,
+                mix: Optional[torch.Tensor] = None, gain: Optional[torch.Tensor] = None, take: Optional[torch.Tensor] = None,
+                weight: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None, eps: float = 0.0,
+                centred: bool = True, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One pass over the streams ``x`` [streams, tokens, width] (32-bit), in up to three parts.  With ``y``: every
+    stream becomes a mix of the old ones plus its share of y, x_t <- sum_s mix[s, t] x_s + gain[t] y, in place.  With
+    ``h``: u = sum_t take[t] x_t (``take`` None: the plain sum) goes to ``h``, normed if ``weight`` is given:
+    (u - mean) / sqrt(var + eps) * weight + bias, or without the mean if not ``centred``.  ``rows`` (int32): output
+    row r reads row rows[r] (not with ``y``).  mix, gain and take are 32-bit."""
+    _dev(x, "x")
+    if x.dim() != 3 or x.dtype != torch.float32:
+        raise KernelError(f"stream_step: x must be float32 [streams, tokens, width], got {x.dtype} {tuple(x.shape)}")
+    streams, tokens, width = x.shape
+    for t, what, count in ((mix, "mix", streams * streams), (gain, "gain", streams), (take, "take", streams)):
+        if t is not None:
+            _dev(t, what)
+            if t.dtype != torch.float32 or t.numel() != count:
+                raise KernelError(f"stream_step: {what} must be float32 with {count} entries")
+    if y is not None:
+        _dev(y, "y")
+        if tuple(y.shape) != (tokens, width) or mix is None or gain is None or rows is not None:
+            raise KernelError("stream_step: an update takes y [tokens, width], mix and gain, and no row list")
+    out_rows = tokens
+    if rows is not None:
+        _dev(rows, "rows")
+        if rows.dtype != torch.int32:
+            raise KernelError("stream_step: rows must be int32")
+        out_rows = rows.numel()
+    if h is not None:
+        _dev(h, "h")
+        if tuple(h.shape) != (out_rows, width):
+            raise KernelError(f"stream_step: h {tuple(h.shape)} against {out_rows} rows of {width}")
+    if weight is not None:
+        _dev(weight, "weight")
+        if weight.numel() != width or (bias is not None and (bias.numel() != width or bias.dtype != weight.dtype)):
+            raise KernelError("stream_step: the norm's weight and bias must have one entry per channel and one type")
+    lib = core()
+    _check(lib, lib.nnis_stream_step(x.data_ptr(), streams, tokens, width, _ptr(y), _code(y) if y is not None else 0, _ptr(mix),
+                                     _ptr(gain), _ptr(take), _ptr(weight), _ptr(bias), _code(weight) if weight is not None else 0,
+                                     1 if centred else 0, float(eps), _ptr(h), _code(h) if h is not None else 0, _ptr(rows),
+                                     out_rows, _stream()))
+    return h
+
+
+def branch_mean(branches, weights, biases, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out = mean over the branches of (y + b) / sqrt(mean((y + b)^2) + eps) * w: up to four inputs [tokens, width]
+    of one type, each with a weight and a bias or None."""
+    count = len(branches)
+    if not 1 <= count <= 4 or len(weights) != count or len(biases) != count:
+        raise KernelError("branch_mean: one to four branches, each with a weight and a bias or None")
+    _dev(out, "out")
+    tokens, width = out.shape
+    for y, w, b in zip(branches, weights, biases):
+        _dev(y, "branch"), _dev(w, "weight")
+        if tuple(y.shape) != (tokens, width) or y.dtype != branches[0].dtype or w.numel() != width or w.dtype != weights[0].dtype:
+            raise KernelError("branch_mean: branches and weights must agree in shape and type")
+        if b is not None:
+            _dev(b, "bias")
+            if b.numel() != width or b.dtype != weights[0].dtype:
+                raise KernelError("branch_mean: a bias has the weights' shape and type")
+    pointers = lambda items: (ctypes.c_void_p * count)(*[None if t is None else t.data_ptr() for t in items])  # noqa: E731
+    ys, ws, bs = pointers(branches), pointers(weights), pointers(biases)
+    lib = core()
+    _check(lib, lib.nnis_branch_mean(ctypes.cast(ys, _VOID), ctypes.cast(ws, _VOID), ctypes.cast(bs, _VOID), count,
+                                     _code(branches[0]), _code(weights[0]), tokens, width, float(eps), out.data_ptr(), _code(out),
+                                     _stream()))
+    return out
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gated_act(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> torch.Tensor:
+    """out = act(gate) * up on a fused [tokens, 2 * inner] projection, gate columns first."""
+    if activation == "silu":
+        return silu_mul(gate_up, out)
+    _dev(gate_up, "gate_up"), _dev(out, "out")
+    tokens, inner = out.shape
+    if gate_up.shape != (tokens, 2 * inner) or activation not in ACTIVATIONS:
+        raise KernelError(f"gated_act: gate_up {tuple(gate_up.shape)} against out {tuple(out.shape)}, activation {activation!r}")
+    lib = core()
+    _check(lib, lib.nnis_gated_act(gate_up.data_ptr(), _code(gate_up), out.data_ptr(), _code(out), tokens, inner,
+                                   ACTIVATIONS[activation], _stream()))
+    return out
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    _dev(y, "y"), _dev(bias, "bias")
+    if y.dim() != 2 or bias.numel() != y.shape[1]:
+        raise KernelError(f"add_bias: a bias of {bias.numel()} for rows of {tuple(y.shape)}")
+    lib = core()
+    _check(lib, lib.nnis_add_bias(y.data_ptr(), _code(y), bias.data_ptr(), _code(bias), y.shape[0], y.shape[1], _stream()))
+    return y
+
+
+# ---------------------------------------------------------------------------
+# mixers that carry state
+# ---------------------------------------------------------------------------
+
+def _step_arrays(ctx, what: str):
+    for t in (ctx.tok_slot, ctx.tok_pos, ctx.seq_slot, ctx.seq_start):
+        _dev(t, "step metadata")
+        if t.dtype != torch.int32:
+            raise KernelError(f"{what}: step metadata must be int32")
+    if ctx.seq_start.numel() < ctx.batch + 1 or ctx.seq_slot.numel() < ctx.batch:
+        raise KernelError(f"{what}: the step's sequence arrays are shorter than its {ctx.batch} sequences")
+
+
+def conv_silu(x: torch.Tensor, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+              ctx, out: torch.Tensor) -> torch.Tensor:
+    """out[t, c] = silu(bias[c] + sum_j weight[c, j] x[t - (taps - 1) + j, c]) over each sequence's own tokens, the
+    last tap on the token itself.  ``x``: [tokens, >= channels], its first ``channels`` columns are taken.
+    ``state`` (float32 [slots, taps - 1, channels]) holds each sequence's last inputs and is brought up to date."""
+    _dev(x, "x"), _dev(weight, "weight"), _dev(out, "out")
+    tokens = x.shape[0]
+    taps = weight.shape[1]
+    if weight.shape[0] != channels or x.shape[1] < channels or tuple(out.shape) != (tokens, channels):
+        raise KernelError(f"conv_silu: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit {channels} channels")
+    if bias is not None and (bias.numel() != channels or bias.dtype != weight.dtype):
+        raise KernelError("conv_silu: the bias has one entry per channel and the weight's type")
+    if taps > 1:
+        _dev(state, "state")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, channels):
+            raise KernelError(f"conv_silu: state must be float32 [slots, {taps - 1}, {channels}], got {tuple(state.shape)}")
+    _step_arrays(ctx, "conv_silu")
+    lib = recurrent()
+    _check(lib, lib.nnis_conv_silu(x.data_ptr(), _code(x), x.stride(0), weight.data_ptr(), _ptr(bias), _code(weight), _ptr(state),
+                                   ctx.tok_slot.data_ptr(), ctx.tok_pos.data_ptr(), ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(),
+                                   tokens, ctx.batch, channels, taps, out.data_ptr(), _code(out), _stream()))
+    return out
+
+
+def selective_scan(x: torch.Tensor, dt_pre: torch.Tensor, bc: torch.Tensor, z: torch.Tensor, A: torch.Tensor, D: torch.Tensor,
+                   dt_bias: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor) -> torch.Tensor:
+    """The diagonal recurrence of a selective scan over each sequence's tokens, from and into ``state`` (float32
+    [slots, channels, states]): dt = softplus(dt_pre + dt_bias); S <- exp(dt A) S + dt x B; out = (S . C + D x) *
+    silu(z).  ``x`` [tokens, channels]; ``dt_pre`` float32 [tokens, channels]; ``bc`` float32 [tokens, 2 * states], B
+    then C; ``z``: a view [tokens, channels] whose rows may be further apart; A, D, dt_bias float32."""
+    tokens, channels = x.shape
+    states = A.shape[1]
+    for t, what in ((x, "x"), (dt_pre, "dt_pre"), (bc, "bc"), (A, "A"), (D, "D"), (dt_bias, "dt_bias"), (state, "state"), (out, "out")):
+        _dev(t, what)
+    for t, what, shape in ((dt_pre, "dt_pre", (tokens, channels)), (bc, "bc", (tokens, 2 * states)), (A, "A", (channels, states)),
+                           (D, "D", (channels,)), (dt_bias, "dt_bias", (channels,))):
+        if t.dtype != torch.float32 or tuple(t.shape) != shape:
+            raise KernelError(f"selective_scan: {what} must be float32 {shape}, got {t.dtype} {tuple(t.shape)}")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (channels, states) or tuple(out.shape) != (tokens, channels):
+        raise KernelError("selective_scan: state must be float32 [slots, channels, states] and out [tokens, channels]")
+    if not z.is_cuda or tuple(z.shape) != (tokens, channels) or z.stride(1) != 1:
+        raise KernelError("selective_scan: z must be [tokens, channels] on the GPU with adjacent columns")
+    _step_arrays(ctx, "selective_scan")
+    lib = recurrent()
+    _check(lib, lib.nnis_selective_scan(x.data_ptr(), _code(x), dt_pre.data_ptr(), bc.data_ptr(), z.data_ptr(), _code(z),
+                                        z.stride(0) if tokens > 1 else channels, A.data_ptr(), D.data_ptr(), dt_bias.data_ptr(),
+                                        state.data_ptr(), ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, channels,
+                                        states, out.data_ptr(), _code(out), _stream()))
+    return out
+
+
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logits: torch.Tensor, tau: float, scale: float,
+             state: torch.Tensor, ctx, heads: int, out: torch.Tensor) -> torch.Tensor:
+    """Gated linear attention over each sequence's tokens, from and into ``state`` (float32 [slots, heads, key
+    channels, value channels]): alpha = sigmoid(decay_logits)^(1 / tau); S <- diag(alpha) S + k v^T; out = S^T
+    (q * scale), raw, float32 [tokens, heads * value channels].  q, k [tokens, heads * key channels] and v are views
+    whose rows may be further apart; ``decay_logits`` float32 [tokens, heads * key channels]."""
+    tokens = q.shape[0]
+    key_dim, value_dim = q.shape[1] // heads, v.shape[1] // heads
+    for t, what in ((q, "q"), (k, "k"), (v, "v")):
+        if not t.is_cuda or t.stride(1) != 1 or t.dtype != q.dtype or t.shape[0] != tokens:
+            raise KernelError(f"gla_scan: {what} must be [tokens, channels] on the GPU with adjacent columns, of one type")
+    if k.shape[1] != heads * key_dim or q.shape[1] != heads * key_dim or v.shape[1] != heads * value_dim:
+        raise KernelError(f"gla_scan: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit {heads} heads")
+    _dev(decay_logits, "decay_logits"), _dev(state, "state"), _dev(out, "out")
+    if decay_logits.dtype != torch.float32 or tuple(decay_logits.shape) != (tokens, heads * key_dim):
+        raise KernelError("gla_scan: decay_logits must be float32 [tokens, heads * key channels]")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, key_dim, value_dim):
+        raise KernelError(f"gla_scan: state must be float32 [slots, {heads}, {key_dim}, {value_dim}], got {tuple(state.shape)}")
+    if out.dtype != torch.float32 or tuple(out.shape) != (tokens, heads * value_dim):
+        raise KernelError("gla_scan: out must be float32 [tokens, heads * value channels]")
+    _step_arrays(ctx, "gla_scan")
+    stride = lambda t: t.stride(0) if tokens > 1 else t.shape[1]  # noqa: E731
+    lib = recurrent()
+    _check(lib, lib.nnis_gla_scan(q.data_ptr(), k.data_ptr(), v.data_ptr(), _code(q), stride(q), stride(k), stride(v),
+                                  decay_logits.data_ptr(), float(tau), float(scale), state.data_ptr(), ctx.seq_slot.data_ptr(),
+                                  ctx.seq_start.data_ptr(), ctx.batch, heads, key_dim, value_dim, out.data_ptr(), _stream()))
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * silu(gate[t, h, :]); ``o`` float32
+    [tokens, heads * dim], ``gate`` a view of that shape whose rows may be further apart, ``weight`` [dim]."""
+    _dev(o, "o"), _dev(weight, "weight"), _dev(out, "out")
+    tokens = o.shape[0]
+    dim = o.shape[1] // heads
+    if o.dtype != torch.float32 or o.shape[1] != heads * dim or weight.numel() != dim or tuple(out.shape) != tuple(o.shape):
+        raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit {heads} heads")
+    if not gate.is_cuda or tuple(gate.shape) != tuple(o.shape) or gate.stride(1) != 1:
+        raise KernelError("head_norm_gate: the gate must be [tokens, heads * dim] on the GPU with adjacent columns")
+    lib = recurrent()
+    _check(lib, lib.nnis_head_norm_gate(o.data_ptr(), gate.data_ptr(), _code(gate), gate.stride(0) if tokens > 1 else gate.shape[1],
+                                        weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), tokens, heads, dim, float(eps),
+                                        _stream()))
     return out

@@ -98,6 +98,9 @@ class DecoderModel:
     # ---- cache ---------------------------------------------------------------
     def cache_requests(self) -> Tuple[List[Tuple[int, Any]], Dict[int, int]]:
         requests, shared = [], {}
+        if getattr(self.embedding, "cache_request", None) is not None:
+            # an embedding that keeps something per sequence (the token before a step's first) has a view of its own
+            requests.append(("embedding", self.embedding.cache_request()))
         for index, entry in enumerate(self.spec.schedule):
             if entry.reads_cache_of is None:
                 requests.append((index, self.layers[entry.layer].cache_request()))
@@ -110,7 +113,10 @@ class DecoderModel:
         """ids: int32 [tokens] on the device; want_rows: int32 indices of the
         packed tokens whose logits are asked for.  Returns float32
         [len(want_rows), vocab]."""
-        x = self.embedding.forward(ids, ctx.tokens, rt)
+        if hasattr(self.embedding, "forward_step"):
+            x = self.embedding.forward_step(ids, ctx, cache.view("embedding"), rt)
+        else:
+            x = self.embedding.forward(ids, ctx.tokens, rt)
         for position in self.positions.values():
             x = position.embed(x, ctx, rt)
         stream = (x, None)

@@ -30,7 +30,7 @@ class ModelSpec:
     architecture: str
     width: int
     vocab_size: int
-    max_positions: int
+    max_positions: Optional[int]  # None: the model names no last position; the cache's size bounds a sequence
     stored_dtype: str  # "float32" or "bfloat16": the type random weights are written in
     embedding: Dict[str, Any]
     positions: Dict[str, Dict[str, Any]]  # named position encodings, built once and shared

@@ -16,4 +16,4 @@ from .base import (  # noqa: F401
     register_part,
     registered_kinds,
 )
-from . import attention, block, embedding, feedforward, norm, rope  # noqa: F401
+from . import attention, block, embedding, feedforward, norm, recurrent, rope  # noqa: F401

@@ -4,6 +4,13 @@
 values come from one fused projection; queries and keys are rotated by the
 position encoding handed in; keys and values go into the cache before the
 scores are taken, so the same code runs whole prompts and single tokens.
+
+Options beyond that formula, each off unless the description names it: biases
+on the four projections; values (and a head's output) of another size than
+the keys (``value_dim``); a scale of the scores other than 1 / sqrt(head_dim);
+scores bent by a cap, s -> softcap * tanh(s / softcap), before the softmax;
+a rotation of the first channels of a head only (the position encoding's
+``rot_dim``).
 """
 
 from __future__ import annotations
@@ -20,10 +27,22 @@ from .linear import Projection
 class CausalSelfAttention(Mixer):
     graph_safe = True
 
-    def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None):
+    def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None,
+                 value_dim=None, scale=None, softcap=None, q_bias=None, k_bias=None, v_bias=None, o_bias=None):
         if heads % kv_heads != 0:
             raise InvalidInput(f"{heads} query heads do not divide into {kv_heads} key/value heads")
         self.width, self.heads, self.kv_heads, self.head_dim = int(width), int(heads), int(kv_heads), int(head_dim)
+        self.value_dim = self.head_dim if value_dim is None else int(value_dim)
+        if self.value_dim <= 0:
+            raise InvalidInput(f"value_dim must be positive, got {value_dim}")
+        self.softcap = 0.0 if not softcap else float(softcap)
+        if self.softcap < 0.0:
+            raise InvalidInput(f"the cap of the scores must be positive, got {softcap}")
+        if (q_bias is None) != (k_bias is None) or (q_bias is None) != (v_bias is None):
+            raise InvalidInput("the projections of queries, keys and values have biases all three or none")
+        self.bias_names = {"q": q_bias, "k": k_bias, "v": v_bias, "o": o_bias}
+        self.qkv_bias = None
+        self.output_bias = None
         self.names = {"q": q, "k": k, "v": v, "o": o}
         self.window = None if not window else int(window)
         self.position = None
@@ -31,38 +50,60 @@ class CausalSelfAttention(Mixer):
             if positions is None or position not in positions:
                 raise InvalidInput(f"attention names position encoding {position!r}, which the model does not define")
             self.position = positions[position]
-        self.scale = 1.0 / math.sqrt(self.head_dim)  # runtime.rs:943
+        self.scale = 1.0 / math.sqrt(self.head_dim) if scale is None else float(scale)  # runtime.rs:943
+        if not self.scale > 0.0:
+            raise InvalidInput(f"the scale of the scores must be positive, got {scale}")
         self.qkv = None
         self.out = None
 
     def tensors(self):
         q_width, kv_width = self.heads * self.head_dim, self.kv_heads * self.head_dim
-        return [
+        v_width, o_width = self.kv_heads * self.value_dim, self.heads * self.value_dim
+        out = [
             TensorSpec(self.names["q"], (q_width, self.width)),
             TensorSpec(self.names["k"], (kv_width, self.width)),
-            TensorSpec(self.names["v"], (kv_width, self.width)),
-            TensorSpec(self.names["o"], (self.width, q_width)),
+            TensorSpec(self.names["v"], (v_width, self.width)),
+            TensorSpec(self.names["o"], (self.width, o_width)),
         ]
+        for key, size in (("q", q_width), ("k", kv_width), ("v", v_width), ("o", self.width)):
+            if self.bias_names[key]:
+                out.append(TensorSpec(self.bias_names[key], (size,)))
+        return out
 
     def bind(self, weights, rt):
         # one projection for queries, keys and values: rows q heads, k heads, v heads
         self.qkv = Projection(torch.cat([weights[self.names["q"]], weights[self.names["k"]], weights[self.names["v"]]], dim=0), rt)
         self.out = Projection(weights[self.names["o"]], rt)
+        if self.bias_names["q"]:
+            self.qkv_bias = torch.cat([weights[self.bias_names[key]] for key in ("q", "k", "v")]).contiguous()
+        if self.bias_names["o"]:
+            self.output_bias = weights[self.bias_names["o"]].contiguous()
 
     def weight_bytes(self):
         return self.qkv.weight_bytes() + self.out.weight_bytes()
 
     def cache_request(self):
-        return KVRequest(self.kv_heads, self.head_dim, self.window)
+        return KVRequest(self.kv_heads, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim)
 
     def check(self, rt):
-        rt.ops.attention_check(self.head_dim)
+        rt.ops.attention_check(self.head_dim, self.value_dim)
+        tables = self.position.rotary() if self.position is not None else None
+        rot_dim = tables.rot_dim if tables is not None else getattr(self.position, "rot_dim", 0)
+        if rot_dim > self.head_dim:
+            raise InvalidInput(f"a rotation of {rot_dim} channels does not fit heads of {self.head_dim}")
 
     def _matrix_cores(self, rt) -> bool:
-        return rt.dtype == torch.bfloat16 and self.head_dim % 16 == 0
+        return rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap)
+
+    @property
+    def _plain(self) -> bool:
+        """The formula without any of the options: what the fused kernels of the projections take."""
+        return self.value_dim == self.head_dim and self.qkv_bias is None
 
     def decode_plan(self, batch, longest, rt):
         # (runs of the keys, waves of a block) of a step of single tokens with these sizes
+        if not self._matrix_cores(rt):
+            return None
         return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.head_dim)
 
     def prompt_plan(self, batch, rows, longest, rt):
@@ -87,7 +128,7 @@ class CausalSelfAttention(Mixer):
         tables = self.position.rotary() if self.position is not None else None
         writes = not view.read_only
         if isinstance(x, PendingNorm):
-            if (x.can_fuse(self.qkv.weight) and tables is not None and tables.rot_dim == self.head_dim
+            if (self._plain and x.can_fuse(self.qkv.weight) and tables is not None and tables.rot_dim == self.head_dim
                     and self.head_dim % 32 == 0 and view.k_pages.dtype == torch.bfloat16):
                 # residual sum, norm, the three projections, the rotation and the cache write in one kernel
                 rope = dict(cos=tables.cos, sin=tables.sin, tok_slot=ctx.tok_slot, tok_pos=ctx.tok_pos,
@@ -105,29 +146,36 @@ class CausalSelfAttention(Mixer):
             tables.cos if tables else None, tables.sin if tables else None, tables.rot_dim if tables else 0,
             ctx.tok_slot, ctx.tok_pos,
             view.k_pages if writes else None, view.v_pages if writes else None, view.block_table if writes else None,
-            self.heads, self.kv_heads, self.head_dim,
+            self.heads, self.kv_heads, self.head_dim, self.value_dim, self.qkv_bias,
         )
         return q
 
-    def forward(self, x, ctx, view, rt, into=None):
+    can_leave_bias = True  # ``forward(..., bias_later=True)`` leaves ``output_bias`` to a consumer that adds it in a kernel of its own
+
+    def forward(self, x, ctx, view, rt, into=None, bias_later=False):
         q = self._project_rotate_store(x, ctx, view, rt)
         tokens = q.shape[0]
-        attn = rt.empty(tokens, self.heads * self.head_dim)
+        attn = rt.empty(tokens, self.heads * self.value_dim)
         # a decode step over long sequences leaves its runs of keys to the output projection, if that takes them
         step = None
-        if ctx.decode and q.dtype == torch.bfloat16:
+        fast = self._matrix_cores(rt) and view.k_pages.dtype == torch.bfloat16
+        if ctx.decode and fast:
             step = ctx.step_tables(rt, self.position.rotary() if self.position is not None else None, view.block_table)
         plan = ctx.options.get("causal_attention")  # (a test or a sweep names the launch; else the sizes choose)
-        if plan is None:
+        if plan is None and fast:
             plan = (self.decode_plan(ctx.batch, ctx.planned_len, rt) if ctx.decode
                     else self.prompt_plan(ctx.batch, ctx.planned_rows, ctx.planned_len, rt))
         attn = rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0,
-                                keep_runs=into is not None, tables=step, plan=plan)
+                                keep_runs=into is not None and self.output_bias is None, tables=step, plan=plan,
+                                value_dim=self.value_dim, softcap=self.softcap)
         if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
             attn = attn.combine()
-        if into is not None and into.can_take(attn, self.out.weight):
+        if into is not None and self.output_bias is None and into.can_take(attn, self.out.weight):
             return into.take(attn, self.out.weight)  # the output projection adds to the stream itself
-        return self.out(attn, rt)
+        y = self.out(attn, rt)
+        if self.output_bias is not None and not bias_later:
+            rt.ops.add_bias(y, self.output_bias)
+        return y
 
 
 register_part("mixer", "causal_attention", CausalSelfAttention)

@@ -56,10 +56,12 @@ class TensorSpec:
     marks a table of integers, uniform in [0, ``high``), which is stored and
     kept as int32 whatever the activation type.  A part may register a rule
     of its own.  ``fallback`` names another checkpoint
-    tensor that stands in when this one is absent (a tied head)."""
+    tensor that stands in when this one is absent (a tied head).  A size in
+    ``shape`` may be None: the part takes whatever the checkpoint has there
+    (a random model cannot be drawn for such a part)."""
 
     name: str
-    shape: Tuple[int, ...]
+    shape: Tuple[Optional[int], ...]
     init: str = "matrix"
     fallback: Optional[str] = None
     high: Optional[int] = None
@@ -181,6 +183,10 @@ class PositionEncoding(Part):
 
     def embed(self, x, ctx, rt):
         return x
+
+    def reach(self, positions: int) -> None:
+        """Told how far the engine's cache lets a sequence grow: an encoding
+        of a model that names no last position sizes its tables by this."""
 
 
 class Mixer(Part):

@@ -15,8 +15,12 @@ second one, or the first of the block that comes next (``following``).
 
 from __future__ import annotations
 
-from .base import Block, build_part, register_part
-from .lazy import PendingNorm, ResidualInto
+import torch
+
+from ..errors import InvalidInput
+from ..weights.random_init import register_init_rule
+from .base import Block, TensorSpec, build_part, register_part
+from .lazy import PendingNorm, PreparedStreams, ResidualInto
 
 
 def _joined(plans):
@@ -98,4 +102,107 @@ class PreNormBlock(Block):
         return self._run(self.feed_forward, normed, (ctx, rt), following, rt)
 
 
+class HyperConnectionBlock(Block):
+    """A pre-norm layer over a residual kept as ``streams`` streams x_1 .. x_s
+    (all equal to the embedding at the start; their sum is the model's output).
+    A sublayer, the mixer or the feed-forward, reads a weighted sum of the
+    streams and writes into all of them:
+
+        u = sum_s take[s] x_s;   y = sublayer(norm(u));   x_t <- sum_s mix[s, t] x_s + gain[t] y
+
+    ``take`` belongs to the norm (a norm over streams reads them itself);
+    ``mix`` [from, to] and ``gain`` are this block's, one pair a sublayer.  The
+    update and the norm that comes next (this block's second, or the first of
+    the block behind it) are one kernel.  Without a feed-forward the layer has
+    the first sublayer only."""
+
+    def __init__(self, width, streams, norm1, mixer, connect1, norm2=None, feed_forward=None, connect2=None, positions=None):
+        self.width, self.streams = int(width), int(streams)
+        if (feed_forward is None) != (norm2 is None) or (feed_forward is None) != (connect2 is None):
+            raise InvalidInput("a feed-forward comes with its norm and its connections, or none of the three")
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer, positions=positions)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        self.connections = [connect1] + ([connect2] if connect2 is not None else [])
+        self._parts = [part for part in (self.norm1, self.mixer, self.norm2, self.feed_forward) if part is not None]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self._parts)
+        self._mix = self._gain = None
+
+    def tensors(self):
+        out = [spec for part in self._parts for spec in part.tensors()]
+        for connect in self.connections:
+            out.append(TensorSpec(connect["mix"], (self.streams, self.streams), init="stream_mix"))
+            out.append(TensorSpec(connect["gain"], (self.streams,), init="stream_share"))
+        return out
+
+    def bind(self, weights, rt):
+        for part in self._parts:
+            part.bind(weights, rt)
+        # the connections' coefficients are kept in 32-bit whatever they are stored in
+        self._mix = [weights[connect["mix"]].float().contiguous() for connect in self.connections]
+        self._gain = [weights[connect["gain"]].float().contiguous() for connect in self.connections]
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for part in self._parts)
+
+    def cache_request(self):
+        return self.mixer.cache_request()
+
+    def check(self, rt):
+        for part in self._parts:
+            part.check(rt)
+        if not 1 <= self.streams <= 8:
+            raise InvalidInput(f"the streams' kernels take 1 to 8 streams, got {self.streams}")
+
+    def decode_plan(self, batch, longest, rt):
+        return _joined(part.decode_plan(batch, longest, rt) for part in self._parts)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        return _joined(part.prompt_plan(batch, rows, longest, rt) for part in self._parts)
+
+    def held_buffers(self, rt):
+        return [buffer for part in self._parts for buffer in part.held_buffers(rt)]
+
+    @property
+    def entry_norm(self):
+        return self.norm1
+
+    def forward(self, stream, ctx, view, rt, following=None):
+        """stream: (x, None) with x [streams, tokens, width], or this block's first
+        norm already run by the block before (``PreparedStreams``).  following: the
+        next block's first norm; if it reads these streams it is run here and handed on."""
+        if isinstance(stream, PreparedStreams):
+            if stream.norm is not self.norm1:
+                raise ValueError("the rows handed to a block are not those of the block's own first norm")
+            x, h = stream.x, stream.h
+        else:
+            x, pending = stream
+            if pending is not None:
+                raise InvalidInput("a block over several streams takes them with nothing left to add")
+            if x.dim() == 2:
+                if self.streams != 1:
+                    raise InvalidInput(f"a block over {self.streams} streams was handed a single one")
+                x = x.unsqueeze(0)
+            h = self.norm1.forward(x, rt)
+        y = self.mixer.forward(h, ctx, view, rt)
+        if self.feed_forward is not None:
+            h = self.norm2.update_forward(x, y, self._mix[0], self._gain[0], rt)
+            y = self.feed_forward.forward(h, ctx, rt)
+        mix, gain = self._mix[-1], self._gain[-1]
+        if following is not None and hasattr(following, "update_forward") and getattr(following, "streams", 0) == self.streams:
+            return PreparedStreams(following, x, following.update_forward(x, y, mix, gain, rt))
+        rt.ops.stream_step(x, y=y, mix=mix, gain=gain)
+        return x, None
+
+
+def _noise(spec, generator):
+    return torch.randn(tuple(spec.shape), generator=generator, dtype=torch.float32)
+
+
+# what a random model draws for the connections: a mix near the identity, shares spread around one half
+register_init_rule("stream_mix", lambda spec, generator, dtype: (torch.eye(spec.shape[0]) + 0.2 * _noise(spec, generator)).to(dtype), replace=True)
+register_init_rule("stream_share", lambda spec, generator, dtype: (0.5 + 0.25 * _noise(spec, generator)).to(dtype), replace=True)
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "hyper_connections", HyperConnectionBlock)

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Part, TensorSpec, register_part
+from .base import Part, StateRequest, TensorSpec, register_part
 from .linear import Projection
 
 
@@ -40,6 +40,39 @@ class TokenEmbedding(Part):
         return rt.ops.embed(ids, self.table, rt.empty(tokens, self.width, dtype=torch.float32))
 
 
+class PairHashEmbedding(Part):
+    """A token's row of the table plus a row of a second table chosen by the
+    token and the one before it: row (before * mul_prev + token * mul_cur) %
+    buckets, and row ``buckets`` (the last) for a sequence's first token.  The
+    token before a step's first is part of the sequence's state: one integer
+    per slot, which the cache keeps (``cache_request``).  ``copies`` > 1 gives
+    the output as that many equal streams ``[copies, tokens, width]``."""
+
+    graph_safe = True
+
+    def __init__(self, vocab_size, width, weight, pairs, buckets, mul_prev, mul_cur, copies=1):
+        self.vocab_size, self.width, self.weight_name, self.pairs_name = int(vocab_size), int(width), weight, pairs
+        self.buckets, self.mul_prev, self.mul_cur, self.copies = int(buckets), int(mul_prev), int(mul_cur), int(copies)
+        self.table = self.pairs = None
+
+    def tensors(self):
+        return [TensorSpec(self.weight_name, (self.vocab_size, self.width)),
+                TensorSpec(self.pairs_name, (self.buckets + 1, self.width))]
+
+    def bind(self, weights, rt):
+        self.table = weights[self.weight_name].contiguous()
+        self.pairs = weights[self.pairs_name].contiguous()
+
+    def cache_request(self):
+        return StateRequest((), "int32")
+
+    def forward_step(self, ids, ctx, view, rt):
+        """ids: int32 on the device -> the 32-bit residual [copies, tokens, width] ([tokens, width] for one copy)."""
+        out = rt.empty(self.copies, ctx.tokens, self.width, dtype=torch.float32)
+        rt.ops.embed_pair(ids, ctx.tok_slot, ctx.tok_pos, self.table, self.pairs, self.mul_prev, self.mul_cur, view.state, out)
+        return out if self.copies > 1 else out[0]
+
+
 class LinearHead(Part):
     graph_safe = True
 
@@ -66,4 +99,5 @@ class LinearHead(Part):
 
 
 register_part("embedding", "table", TokenEmbedding)
+register_part("embedding", "table_pairs", PairHashEmbedding)
 register_part("head", "linear", LinearHead)

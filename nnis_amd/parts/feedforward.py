@@ -1,7 +1,8 @@
 """Gated feed-forward: down( act(gate x) * up x ), act = SiLU
 (/root/reference/crates/nnis-model/src/runtime.rs:1054-1087;
-/root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28).  Gate and up are
-one fused projection whose first ``inner`` output columns are the gate."""
+/root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28) or the tanh form
+of GELU.  Gate and up are one fused projection whose first ``inner`` output
+columns are the gate."""
 
 from __future__ import annotations
 
@@ -16,8 +17,9 @@ class GatedFeedForward(FeedForward):
     graph_safe = True
 
     def __init__(self, width, inner, gate, up, down, activation="silu"):
-        if activation != "silu":
-            raise Unsupported(f"gated feed-forward activation {activation!r}; only silu is built")
+        if activation not in ("silu", "gelu_tanh"):
+            raise Unsupported(f"gated feed-forward activation {activation!r}; silu and gelu_tanh are built")
+        self.activation = activation
         self.width, self.inner = int(width), int(inner)
         self.names = {"gate": gate, "up": up, "down": down}
         self.gate_up = None
@@ -43,14 +45,14 @@ class GatedFeedForward(FeedForward):
     def forward(self, x, ctx, rt, into=None):
         from .lazy import PendingNorm
 
-        if isinstance(x, PendingNorm) and x.can_fuse(self.gate_up.weight):
+        if isinstance(x, PendingNorm) and self.activation == "silu" and x.can_fuse(self.gate_up.weight):
             # (residual sum,) norm, both projections and the gating in one kernel
             hidden = x.fused(self.gate_up.weight, rt.empty(x.rows, self.inner), rt.ops.EPILOGUE_SILU)
         else:
             if isinstance(x, PendingNorm):
                 x = x.materialize()
             gate_up = self.gate_up(x, rt)
-            hidden = rt.ops.silu_mul(gate_up, rt.empty(x.shape[0], self.inner))
+            hidden = rt.ops.gated_act(gate_up, rt.empty(x.shape[0], self.inner), self.activation)
         if into is not None and into.can_take(hidden, self.down.weight):
             return into.take(hidden, self.down.weight)  # the down projection adds to the stream itself
         return self.down(hidden, rt)

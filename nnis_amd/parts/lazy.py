@@ -106,3 +106,13 @@ class ResidualInto:
         ss = rt.empty(rt.ops.gemm_residual_parts(rows, width), rows, dtype=torch.float32)
         parts = rt.ops.gemm_residual(x, weight, residual, self.norm.weight, scaled, ss)
         return PendingNorm.prepared(self.norm, residual, scaled, ss, parts, rt)
+
+
+class PreparedStreams:
+    """What a block over several residual streams hands the block that comes
+    next when it has run that block's first norm already (in the kernel that
+    brought its own last output into the streams): the streams ``x``
+    [streams, tokens, width] and ``h``, the rows that ``norm`` makes of them."""
+
+    def __init__(self, norm, x: torch.Tensor, h: torch.Tensor):
+        self.norm, self.x, self.h = norm, x, h

@@ -37,3 +37,63 @@ class RMSNorm(Norm):
 
 
 register_part("norm", "rms", RMSNorm)
+
+
+class LayerNorm(Norm):
+    """Layer norm with weight and bias: (x - mean) / sqrt(var + eps) * w + b, the
+    variance being the mean squared deviation; ``centred=False`` leaves the mean
+    in (an RMS norm, then with an optional bias).
+
+    It also reads a residual kept as several streams ``[streams, tokens,
+    width]``: what it norms is then u = sum_s take[s] x_s, ``take`` a tensor of
+    the checkpoint, or the plain sum of the streams without one.  The streams'
+    update by the sublayer before (``update_forward``) runs in the same kernel."""
+
+    graph_safe = True
+
+    def __init__(self, width: int, eps: float, weight: str, bias: str = None, centred: bool = True, streams: int = 1,
+                 take: str = None):
+        self.width, self.eps, self.centred, self.streams = int(width), float(eps), bool(centred), int(streams)
+        self.weight_name, self.bias_name, self.take_name = weight, bias, take
+        self.weight = self.bias = self.take = None
+
+    def tensors(self):
+        out = [TensorSpec(self.weight_name, (self.width,), init="gain")]
+        if self.bias_name:
+            out.append(TensorSpec(self.bias_name, (self.width,)))
+        if self.take_name:
+            out.append(TensorSpec(self.take_name, (self.streams,), init="stream_share"))
+        return out
+
+    def bind(self, weights, rt):
+        self.weight = weights[self.weight_name].contiguous()
+        self.bias = weights[self.bias_name].contiguous() if self.bias_name else None
+        self.take = weights[self.take_name].float().contiguous() if self.take_name else None  # (the coefficients are kept in 32-bit)
+
+    def weight_bytes(self):
+        return sum(t.numel() * t.element_size() for t in (self.weight, self.bias) if t is not None)
+
+    def _streams(self, x):
+        return x if x.dim() == 3 else x.unsqueeze(0)
+
+    def forward(self, x, rt, rows=None):
+        count = x.shape[-2] if rows is None else rows.shape[0]
+        return rt.ops.stream_step(self._streams(x), rt.empty(count, self.width), take=self.take, weight=self.weight, bias=self.bias,
+                                  eps=self.eps, centred=self.centred, rows=rows)
+
+    def update_forward(self, x, y, mix, gain, rt):
+        """x_t <- sum_s mix[s, t] x_s + gain[t] y for every stream, in place, and then this norm of the new streams."""
+        return rt.ops.stream_step(x, rt.empty(x.shape[-2], self.width), y=y, mix=mix, gain=gain, take=self.take, weight=self.weight,
+                                  bias=self.bias, eps=self.eps, centred=self.centred)
+
+    def add_forward(self, residual, delta, rt, rows=None):
+        import torch
+
+        one = torch.ones(1, dtype=torch.float32, device=residual.device)
+        if rows is None:
+            return self.update_forward(self._streams(residual), delta, one, one, rt)
+        rt.ops.stream_step(self._streams(residual), y=delta, mix=one, gain=one)
+        return self.forward(residual, rt, rows=rows)
+
+
+register_part("norm", "layer", LayerNorm)

@@ -14,8 +14,16 @@ from ..errors import InvalidInput
 from .base import PositionEncoding, RotaryTables, register_part
 
 
-def rotary_tables(positions: int, rot_dim: int, theta: float):
+def rotary_tables(positions: int, rot_dim: int, theta: float, angles: str = "float32"):
+    """``angles``: "float32" rounds the frequencies and the angles to 32-bit as
+    the reference does; "float64" takes frequency i as theta^(-2i / rot_dim) and
+    the angle as position x frequency in 64-bit, and rounds cosine and sine only."""
     half = rot_dim // 2
+    if angles == "float64":
+        pair = torch.arange(half, dtype=torch.float64)
+        inv_freq = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * pair / float(rot_dim))
+        angle = torch.arange(positions, dtype=torch.float64)[:, None] * inv_freq[None, :]
+        return torch.cos(angle).to(torch.float32), torch.sin(angle).to(torch.float32)
     pair = torch.arange(half, dtype=torch.float32)
     exponent = (2.0 * pair) / torch.tensor(float(rot_dim), dtype=torch.float32)  # 32-bit quotient
     theta32 = torch.tensor(theta, dtype=torch.float32).to(torch.float64)
@@ -30,17 +38,35 @@ def rotary_tables(positions: int, rot_dim: int, theta: float):
 class RotaryHalf(PositionEncoding):
     graph_safe = True
 
-    def __init__(self, rot_dim: int, theta: float, max_positions: int):
+    def __init__(self, rot_dim: int, theta: float, max_positions: int = None, angles: str = "float32"):
+        """``max_positions`` None: the model names no last position; the tables
+        are made as long as the engine's cache lets a sequence grow (``reach``)."""
         if rot_dim <= 0 or rot_dim % 2 != 0:
             raise InvalidInput(f"rotary dimension must be even and positive; got {rot_dim}")
+        if angles not in ("float32", "float64"):
+            raise InvalidInput(f"rotary angles are made in float32 or float64, got {angles!r}")
         self.rot_dim = int(rot_dim)
         self.theta = float(theta)
-        self.max_positions = int(max_positions)
+        self.max_positions = None if max_positions is None else int(max_positions)
+        self.angles = angles
         self._tables = None
+        self._device = None
+        self._kept = []
 
     def bind(self, weights, rt):
-        cos, sin = rotary_tables(self.max_positions, self.rot_dim, self.theta)
-        self._tables = RotaryTables(cos.to(rt.device).contiguous(), sin.to(rt.device).contiguous(), self.rot_dim)
+        self._device = rt.device
+        self._make(self.max_positions or 64)
+
+    def _make(self, positions: int) -> None:
+        cos, sin = rotary_tables(positions, self.rot_dim, self.theta, self.angles)
+        self._tables = RotaryTables(cos.to(self._device).contiguous(), sin.to(self._device).contiguous(), self.rot_dim)
+
+    def reach(self, positions: int) -> None:
+        """Makes the tables cover ``positions`` positions, if the model sets no end of its own.  Called when an
+        engine is made, before any step is captured: captured steps hold the tables' addresses."""
+        if self.max_positions is None and self._tables is not None and self._tables.cos.shape[0] < positions:
+            self._kept.append(self._tables)  # (steps captured by an earlier engine of the same model go on reading these)
+            self._make(positions)
 
     def rotary(self):
         return self._tables

@@ -120,7 +120,8 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
             continue
         consumed.add(source)
         stored, shape = where[source].entries[source]
-        if tuple(shape) != tuple(spec.shape):
+        if len(shape) != len(spec.shape) or any(want is not None and want != have for want, have in zip(spec.shape, shape)):
+            # (a size that a part leaves open, None, is whatever the file has)
             wrong_shape.append(f"{source}: expected {list(spec.shape)}, file has {list(shape)}")
             continue
         if spec.init == "index":

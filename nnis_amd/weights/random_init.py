@@ -72,6 +72,9 @@ def write_random_model(model_dir: str, raw_config: Dict[str, Any], seed: int) ->
             if tensor.name in done or tensor.fallback is not None:
                 continue  # a tensor with a stand-in (tied head) is not drawn
             done.add(tensor.name)
+            if any(size is None for size in tensor.shape):
+                raise InvalidInput(f"tensor {tensor.name}: the model leaves a size open ({list(tensor.shape)}); a random model "
+                                   "needs every size in its configuration")
             rule = _INIT_RULES.get(tensor.init)
             if rule is None:
                 raise InvalidInput(f"tensor {tensor.name}: unknown init rule {tensor.init!r}; registered: "

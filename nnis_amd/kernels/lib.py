@@ -49,7 +49,7 @@ FLAGS = [
 # in scratch memory, all outside their loops over the keys; no other kernel of either file spills.)
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
-PREBUILT_WIDE_VALUES = ("attn_hd32v64", "attn_hd64v128", "attn_hd16v48")  # values of another size than the keys: what the tests use
+PREBUILT_WIDE_VALUES = ("attn_hd32v64", "attn_hd64v32", "attn_hd16v48")  # values of another size than the keys: what the tests use
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

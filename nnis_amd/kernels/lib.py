@@ -48,8 +48,9 @@ FLAGS = [
 # sums in vector registers the prefill attention's four-column kernels at 64 channels keep 17 to 26 registers
 # in scratch memory, all outside their loops over the keys; no other kernel of either file spills.)
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
-PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
-PREBUILT_WIDE_VALUES = ("attn_hd32v64", "attn_hd64v32", "attn_hd16v48")  # values of another size than the keys: what the tests use
+PREBUILT_HEAD_DIMS = (6, 16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
+# values of another size than the keys: what the tests use
+PREBUILT_WIDE_VALUES = ("attn_hd32v16", "attn_hd16v48", "attn_hd48v64", "attn_hd64v32", "attn_hd6v10")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -1,0 +1,470 @@
+"""Zifunex on the GPU against the plain implementation (``plain_zifunex``):
+each mechanism alone, then whole models through the engine -- prompts whole, in
+portions and token by token, unequal batches, slots and pages used again, keys
+far away and at page borders, long decoding, greedy generation through the
+library's entry point.  32-bit is held to rounding; bfloat16 to the error of
+the plain model run with its activations rounded where the engine rounds them.
+"""
+
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+import nnis_amd
+import plain_zifunex as Z
+from gpu_helpers import cache_for, context, runtime
+from zifunex_configs import ZIFUNEX_CONFIGS, attention, gla, parallel, scan, zifunex
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+HEAD_SIZES = [(32, 16), (16, 48), (48, 64), (64, 32), (32, 32), (64, 64), (16, 16), (6, 10)]  # (key, value) channels of a head
+
+
+def _relative(got, want):
+    got, want = torch.as_tensor(np.asarray(got)).double(), torch.as_tensor(np.asarray(want)).double()
+    return float((got - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt().clamp_min(1e-30))
+
+
+def _close(got, want, dtype, what="", bf16=3e-2):
+    """Root mean square of the difference over that of the values: 32-bit rounding, or bfloat16's."""
+    error = _relative(got.detach().float().cpu() if isinstance(got, torch.Tensor) else got, want)
+    bound = 3e-5 if dtype == "float32" else bf16
+    assert error <= bound, f"{what}: relative error {error:.3g} (bound {bound:.3g})"
+
+
+def _weights(mixer, dtype, seed, scale=None):
+    """Random tensors for a part, by its own declarations; returns (for the plain functions in 64-bit, for the part)."""
+    from nnis_amd.weights.random_init import _INIT_RULES
+
+    generator = torch.Generator().manual_seed(seed)
+    stored = {}
+    for t in mixer.tensors():
+        value = _INIT_RULES[t.init](t, generator, torch.bfloat16)
+        if scale and t.name in scale:
+            value = (value.float() * scale[t.name]).to(torch.bfloat16)
+        stored[t.name] = value
+    wide = torch.float32 if dtype == "float32" else torch.bfloat16
+    return {n: v.double() for n, v in stored.items()}, {n: v.to(wide).cuda() for n, v in stored.items()}
+
+
+def _run_in_steps(mixer, cache, rt, xs, cuts):
+    """Runs sequences (rows of ``xs``) through a mixer, all of them in every step: ``cuts[i]`` lists where sequence i's
+    portions end.  Returns each sequence's outputs, put together."""
+    slots = [cache.acquire() for _ in xs]
+    done = [0] * len(xs)
+    outs = [[] for _ in xs]
+    cuts = [list(c) for c in cuts]
+    while any(cuts):
+        batch = [i for i in range(len(xs)) if cuts[i]]
+        ends = [cuts[i].pop(0) for i in batch]
+        ctx = context(cache, [(slots[i], end - done[i]) for i, end in zip(batch, ends)])
+        x = torch.cat([xs[i][done[i]:end] for i, end in zip(batch, ends)]).to(rt.dtype).cuda()
+        y = mixer.forward(x, ctx, cache.view(0), rt)
+        row = 0
+        for i, end in zip(batch, ends):
+            outs[i].append(y[row:row + end - done[i]].float().cpu())
+            row += end - done[i]
+            done[i] = end
+    for slot in slots:
+        cache.release(slot)
+    return [torch.cat(o) for o in outs]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim, rot, width", [(4, 2, 32, 16, 16, 64), (2, 1, 16, 48, 16, 48), (6, 1, 48, 64, 24, 96),
+                                                                   (2, 2, 32, 32, 32, 40)])
+def test_capped_attention_alone(dtype, heads, kv_heads, dim, vdim, rot, width):
+    """Biases, grouped heads, values of their own size, part of a head rotated, a cap on the scores.  The queries'
+    and keys' weights are large enough for the cap to bend most scores."""
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    sizes = attention(heads, kv_heads, dim, vdim, rot, base=777.0, scale=0.3, softcap=6.0)
+    rope = build_part("position", {"kind": "rotary_half", "rot_dim": rot, "theta": 777.0, "max_positions": None, "angles": "float64"})
+    rope.bind({}, rt)
+    rope.reach(512)
+    names = {k: k for k in ("q", "k", "v", "o")}
+    mixer = build_part("mixer", dict(kind="causal_attention", width=width, heads=heads, kv_heads=kv_heads, head_dim=dim, value_dim=vdim,
+                                     scale=0.3, softcap=6.0, position="r", q_bias="q.b", k_bias="k.b", v_bias="v.b", o_bias="o.b", **names),
+                       positions={"r": rope})
+    plain_w, part_w = _weights(mixer, dtype, 3, scale={"q": 30.0, "k": 30.0, "q.b": 20.0, "k.b": 20.0, "v.b": 20.0, "o.b": 20.0})
+    mixer.bind(part_w, rt)
+    cache = cache_for([mixer.cache_request()], rt, max_tokens=1024, max_positions=512)
+    generator = torch.Generator().manual_seed(5)
+    lengths = [150, 3, 67]
+    xs = [torch.randn(n, width, generator=generator).to(torch.bfloat16).double() for n in lengths]
+    rnd = Z.identity if dtype == "float32" else Z.bf16_round
+    want = [Z.capped_attention(x, plain_w, sizes, rnd) for x in xs]
+    scores_bent = float((xs[0] @ plain_w["q"].T).abs().mean()) * float((xs[0] @ plain_w["k"].T).abs().mean()) * 0.3
+    assert scores_bent > 1.0
+    # whole; then a prompt, portions down to two tokens and single tokens, across page borders (64, 128)
+    for cuts in ([[150], [3], [67]], [[61, 63, 64, 66, 128, 130, 131, 150], [1, 2, 3], [2, 4, 64, 65, 66, 67]]):
+        got = _run_in_steps(mixer, cache, rt, xs, cuts)
+        for g, w, n in zip(got, want, lengths):
+            _close(g, w, dtype, f"attention {cuts[0][:2]} length {n}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_and_the_first_key_count(dtype):
+    """One query matches one key far back, across several pages: the output there is that key's value.  Leaving
+    the key out (a page lost, a run of keys skipped) changes the result by its own size."""
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    width, dim, vdim = 32, 32, 16
+    sizes = attention(1, 1, dim, vdim, 8, base=100.0, scale=1.0, softcap=40.0)
+    rope = build_part("position", {"kind": "rotary_half", "rot_dim": 8, "theta": 100.0, "max_positions": None, "angles": "float64"})
+    rope.bind({}, rt)
+    rope.reach(1024)
+    mixer = build_part("mixer", dict(kind="causal_attention", width=width, heads=1, kv_heads=1, head_dim=dim, value_dim=vdim, scale=1.0,
+                                     softcap=40.0, position="r", q="q", k="k", v="v", o="o", q_bias="q.b", k_bias="k.b", v_bias="v.b",
+                                     o_bias="o.b"), positions={"r": rope})
+    plain_w, part_w = _weights(mixer, dtype, 9)
+    # queries and keys read the input's channels 8..31 as they are (the unrotated part of the head): a query and a key agree where the inputs do
+    eye = torch.zeros(dim, width, dtype=torch.float64)
+    eye[8:, 8:] = torch.eye(24, dtype=torch.float64)
+    for name in ("q", "k"):
+        plain_w[name] = eye.clone()
+        part_w[name] = eye.to(part_w[name].dtype).cuda()
+        plain_w[name + ".b"].zero_()
+        part_w[name + ".b"].zero_()
+    mixer.bind(part_w, rt)
+    cache = cache_for([mixer.cache_request()], rt, max_tokens=2048, max_positions=1024)
+    n = 700
+    generator = torch.Generator().manual_seed(1)
+    for far in (0, 1, 63, 64, 500):
+        x = (0.05 * torch.randn(n, width, generator=generator)).to(torch.bfloat16).double()
+        mark = torch.zeros(width, dtype=torch.float64)
+        mark[8:] = torch.tensor([1.0, -1.0] * 12, dtype=torch.float64) * 1.5  # 24 x 2.25 = 54 > the cap: that score sits at the cap's end
+        x[far] = mark
+        x[n - 1] = mark
+        # (the two agree for queries and keys only: their values, which read all channels, differ)
+        x[far, :8] = (2.0 * torch.randn(8, generator=generator)).to(torch.bfloat16).double()
+        x[n - 1, :8] = (2.0 * torch.randn(8, generator=generator)).to(torch.bfloat16).double()
+        x[n - 2] = -mark  # the token before the last must not take its place
+        want = Z.capped_attention(x, plain_w, sizes, Z.identity if dtype == "float32" else Z.bf16_round)
+        without = Z.capped_attention(torch.cat([x[:far], x[far + 1:]]), plain_w, sizes)
+        assert _relative(without[-1], want[-1]) > 0.1  # the far key matters
+        for cuts in ([n], [n - 1, n], [n - 40] + list(range(n - 39, n + 1))):
+            got = _run_in_steps(mixer, cache, rt, [x], [cuts])[0]
+            _close(got[-1], want[-1], dtype, f"far key at {far}, cuts {cuts[:2]}")
+            _close(got, want, dtype, f"far key at {far}, all rows, cuts {cuts[:2]}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("channels, states, dt_rank, taps, width", [(80, 12, 5, 3, 64), (48, 40, 3, 5, 32), (64, 8, 8, 2, 48), (40, 100, 4, 1, 24),
+                                                                   (300, 16, 16, 4, 64)])
+def test_selective_scan_alone(dtype, channels, states, dt_rank, taps, width):
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    names = dict(w_in="in", conv="conv", conv_bias="conv.b", w_x="x", w_dt="dt", dt_bias="dt.b", a_log="A_log", d="D", w_out="o")
+    mixer = build_part("mixer", dict(kind="selective_scan", width=width, channels=channels, states=states, dt_rank=dt_rank, taps=taps, **names))
+    # (small steps: the state still holds the first tokens at the end)
+    plain_w, part_w = _weights(mixer, dtype, 4, scale={"in": 20.0, "x": 20.0, "dt.b": 2.5, "dt": 0.2})
+    mixer.bind(part_w, rt)
+    cache = cache_for([mixer.cache_request()], rt, max_tokens=1024, max_positions=512)
+    generator = torch.Generator().manual_seed(6)
+    lengths = [90, 1, 17]
+    xs = [torch.randn(n, width, generator=generator).to(torch.bfloat16).double() for n in lengths]
+    sizes = scan(channels, states, dt_rank, taps)
+    want = [Z.selective_scan(x, plain_w, sizes, Z.identity if dtype == "float32" else Z.bf16_round) for x in xs]
+    assert float(want[0][-1].abs().max()) > 1e-3
+    # the state carries far: dropping the first token changes the last output
+    assert _relative(Z.selective_scan(xs[0][1:], plain_w, sizes)[-1], Z.selective_scan(xs[0], plain_w, sizes)[-1]) > 1e-4
+    for cuts in ([[90], [1], [17]], [[1, 2, 3, 5, 6, 64, 66, 88, 89, 90], [1], [2, 4, 5, 6, 7, 17]], [list(range(1, 91)), [1], list(range(1, 18))]):
+        got = _run_in_steps(mixer, cache, rt, xs, cuts)
+        for g, w, n in zip(got, want, lengths):
+            _close(g, w, dtype, f"scan length {n} in {len(cuts[0])} steps")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, dim, vdim, tau, rank, width", [(3, 16, 24, 8.0, 8, 64), (2, 40, 20, 1.0, 16, 48), (1, 64, 128, 32.0, 24, 96),
+                                                                (2, 130, 70, 4.0, 8, 32)])
+def test_gated_linear_attention_alone(dtype, heads, dim, vdim, tau, rank, width):
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    names = dict(q="q", k="k", v="v", g="g", o="o", norm="norm", a1="a1", a2="a2", a2_bias="a2.b")
+    mixer = build_part("mixer", dict(kind="gated_linear_attention", width=width, heads=heads, key_dim=dim, value_dim=vdim, tau=tau, eps=1e-5,
+                                     decay_rank=rank, **names))
+    plain_w, part_w = _weights(mixer, dtype, 8, scale={"a1": 5.0, "a2": 5.0, "g": 20.0})
+    mixer.bind(part_w, rt)
+    cache = cache_for([mixer.cache_request()], rt, max_tokens=1024, max_positions=512)
+    generator = torch.Generator().manual_seed(2)
+    lengths = [100, 2, 33]
+    xs = [torch.randn(n, width, generator=generator).to(torch.bfloat16).double() for n in lengths]
+    sizes = {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau}
+    want = [Z.gated_linear_attention(x, plain_w, sizes, 1e-5, Z.identity if dtype == "float32" else Z.bf16_round) for x in xs]
+    if tau >= 4.0:  # the first token is still in the state
+        assert _relative(Z.gated_linear_attention(xs[0][1:], plain_w, sizes, 1e-5)[-1], Z.gated_linear_attention(xs[0], plain_w, sizes, 1e-5)[-1]) > 1e-3
+    for cuts in ([[100], [2], [33]], [[2, 4, 31, 32, 33, 64, 65, 98, 100], [1, 2], [3, 33]], [list(range(1, 101)), [1, 2], list(range(1, 34))]):
+        got = _run_in_steps(mixer, cache, rt, xs, cuts)
+        for g, w, n in zip(got, want, lengths):
+            _close(g, w, dtype, f"gated linear attention length {n} in {len(cuts[0])} steps")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("streams, width", [(1, 40), (3, 96), (8, 520)])
+def test_streams_and_their_norm(dtype, streams, width):
+    """The update of all streams at once from the old ones (mix indexed [from, to]), the weighted sum, the layer norm
+    with bias; a row list; an update without a norm."""
+    rt = runtime(dtype)
+    ops = rt.ops
+    g = torch.Generator().manual_seed(streams)
+    tokens = 37
+    x = torch.randn(streams, tokens, width, generator=g)
+    y = torch.randn(tokens, width, generator=g).to(rt.dtype)
+    mix, gain, take = torch.randn(streams, streams, generator=g), torch.randn(streams, generator=g), torch.randn(streams, generator=g)
+    w, b = (1 + 0.1 * torch.randn(width, generator=g)).to(rt.dtype), (0.1 * torch.randn(width, generator=g)).to(rt.dtype)
+    p = {"in": take.double(), "mix": mix.double(), "out": gain.double()}
+    new = Z.hyper_sublayer(x.double(), p, lambda u: y.double())
+    want = Z.layer_norm(torch.einsum("s,stw->tw", take.double(), new), w.double(), b.double(), 1e-5)
+    dev = x.cuda()
+    h = ops.stream_step(dev, torch.empty(tokens, width, dtype=rt.dtype, device="cuda"), y=y.cuda(), mix=mix.cuda(), gain=gain.cuda(),
+                        take=take.cuda(), weight=w.cuda(), bias=b.cuda(), eps=1e-5)
+    assert _relative(dev.cpu(), new) < 1e-6
+    _close(h, want, dtype, "update and norm", bf16=6e-3)
+    rows = torch.tensor([5, 0, 36, 5], dtype=torch.int32)
+    summed = ops.stream_step(dev, torch.empty(4, width, dtype=rt.dtype, device="cuda"), weight=w.cuda(), bias=b.cuda(), eps=1e-5, rows=rows.cuda())
+    _close(summed, Z.layer_norm(new.sum(dim=0), w.double(), b.double(), 1e-5)[rows.long()], dtype, "plain sum with a row list", bf16=6e-3)
+    before = dev.clone()
+    ops.stream_step(dev, y=y.cuda(), mix=torch.eye(streams).cuda(), gain=torch.zeros(streams).cuda())
+    assert torch.equal(dev, before)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pair_hash_embedding(dtype):
+    """The first token of a sequence takes the table's last row; a token at the start of a later step takes the row
+    of the token that ended the step before, kept per slot; a slot used again starts anew."""
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    part = build_part("embedding", {"kind": "table_pairs", "vocab_size": 50, "width": 24, "weight": "embed", "pairs": "bigram", "buckets": 13,
+                                    "mul_prev": 1000003, "mul_cur": 999983, "copies": 3})
+    g = torch.Generator().manual_seed(0)
+    table, pairs = torch.randn(50, 24, generator=g).to(torch.bfloat16), torch.randn(14, 24, generator=g).to(torch.bfloat16)
+    wide = torch.float32 if dtype == "float32" else torch.bfloat16
+    part.bind({"embed": table.to(wide).cuda(), "bigram": pairs.to(wide).cuda()}, rt)
+    cache = cache_for([part.cache_request()], rt)
+
+    def plain(ids):
+        rows = Z.bigram_rows(ids, 13, 1000003, 999983)
+        return table.float()[torch.tensor(ids)] + pairs.float()[torch.tensor(rows)]
+
+    a, b = [49, 3, 3, 17, 0, 49, 48], [7, 49]
+    sa, sb = cache.acquire(), cache.acquire()
+    steps = [[(sa, a[:3]), (sb, b[:1])], [(sb, b[1:]), (sa, a[3:4])], [(sa, a[4:])]]
+    got = {sa: [], sb: []}
+    for step in steps:
+        ctx = context(cache, [(slot, len(ids)) for slot, ids in step])
+        ids = torch.tensor([t for _, part_ids in step for t in part_ids], dtype=torch.int32).cuda()
+        out = part.forward_step(ids, ctx, cache.view(0), rt)
+        assert out.shape == (3, ids.numel(), 24) and torch.equal(out[0], out[1]) and torch.equal(out[0], out[2])
+        row = 0
+        for slot, part_ids in step:
+            got[slot].append(out[0, row:row + len(part_ids)].cpu())
+            row += len(part_ids)
+    assert torch.allclose(torch.cat(got[sa]), plain(a), atol=1e-6) and torch.allclose(torch.cat(got[sb]), plain(b), atol=1e-6)
+    cache.release(sa)
+    again = cache.acquire()
+    assert again == sa
+    ctx = context(cache, [(again, 2)])
+    out = part.forward_step(torch.tensor([3, 3], dtype=torch.int32).cuda(), ctx, cache.view(0), rt)
+    assert torch.allclose(out[0].cpu(), plain([3, 3]), atol=1e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# whole models through the engine
+# ---------------------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    """Random models of the small configurations.  The queries' and keys' weights and biases are scaled up, so that
+    attention is sharp (a key left out or one too many shows), and so are the decays' and gates' projections."""
+    out = {}
+    for name, (config, seed) in ZIFUNEX_CONFIGS.items():
+        folder = str(tmp_path_factory.mktemp(f"zifunex_{name}"))
+        nnis_amd.write_random_model(folder, config, seed)
+        path = os.path.join(folder, "model.safetensors")
+        tensors = load_file(path)
+        for key in tensors:
+            if key.endswith((".left.q", ".left.k", ".mix.a1", ".mix.a2", ".right.in", ".right.x")):
+                tensors[key] = (tensors[key].float() * 25.0).to(torch.bfloat16)
+            elif key.endswith((".q.b", ".k.b", ".v.b", ".o.b", ".conv.b")) or key in ("embed", "bigram"):
+                tensors[key] = (tensors[key].float() * 20.0).to(torch.bfloat16)
+        save_file(tensors, path)
+        out[name] = folder
+    return out
+
+
+def _ids(count, vocab, seed):
+    generator = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (count,), generator=generator).tolist()
+
+
+class Yardstick:
+    """What the engine may differ from the plain 64-bit logits by, as root mean square relative to the logits' own: in
+    32-bit, rounding; in bfloat16, three times what rounding the plain model's activations to bfloat16 does on the same
+    tokens (a single position: four times the worst position's)."""
+
+    def __init__(self, plain):
+        self.plain, self.known = plain, {}
+        # (a sequence of a few tokens says little about rounding: no bound lies below that of a longer one)
+        self.least = (0.0, 0.0)
+        self.least = self.twin(_ids(64, plain.config["vocab"], 999))[1:]
+
+    def twin(self, ids):
+        key = tuple(ids)
+        if key not in self.known:
+            want, twin = self.plain.logits(ids), self.plain.logits(ids, Z.bf16_round)
+            rows = [_relative(twin[i], want[i]) for i in range(len(ids))]
+            self.known[key] = (want, _relative(twin, want), max(rows))
+            assert 1e-4 < self.known[key][1] < 0.3, self.known[key][1]
+        return self.known[key]
+
+    def check(self, got, ids, dtype, what, rows=None):
+        """``got``: the engine's logits at the positions ``rows`` of the sequence ``ids`` (None: all; an int: that one)."""
+        want, overall, worst = self.twin(ids)
+        single = isinstance(rows, int)
+        want = want if rows is None else want[rows]
+        error = _relative(got, want)
+        bound = 5e-5 if dtype == "float32" else (4.0 * max(worst, self.least[1]) if single else 3.0 * max(overall, self.least[0]))
+        assert error <= bound, f"{what}: relative error {error:.3g} (bound {bound:.3g})"
+
+
+def _collect(engine, slot, ids, cuts):
+    from nnis_amd.engine.batch import StepEntry
+
+    rows, done = [], 0
+    for end in cuts:
+        rows.append(engine.step([StepEntry(slot, ids[done:end], list(range(end - done)))]).cpu())
+        done = end
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(ZIFUNEX_CONFIGS))
+def test_prompts_whole_in_portions_and_token_by_token(folders, name, dtype):
+    config = ZIFUNEX_CONFIGS[name][0]
+    plain = Z.PlainZifunex(folders[name])
+    engine = nnis_amd.load_engine(folders[name], dtype=dtype, max_tokens=1024)
+    ids = _ids(150, config["vocab"], 1)
+    yard = Yardstick(plain)
+    for cuts in ([150], [2, 4, 5, 63, 64, 66, 128, 129, 150], [100] + list(range(101, 151)), list(range(1, 41))):
+        slot = engine.start_sequence()
+        got = _collect(engine, slot, ids, cuts)
+        engine.end_sequence(slot)
+        yard.check(got, ids, dtype, f"{name} cuts {cuts[:3]}..", rows=slice(0, cuts[-1]))
+        # every position by itself, the first tokens among them
+        for place in (0, 1, 2, cuts[-1] - 1):
+            yard.check(got[place], ids, dtype, f"{name} cuts {cuts[:3]}.. position {place}", rows=place)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_unequal_batches_equal_each_request_alone(folders, name, dtype):
+    """Requests of different lengths start together, are decoded together and end one after the other; their slots
+    and pages go to requests that start later.  Every logit equals the plain model's on that request alone."""
+    from nnis_amd.engine.batch import StepEntry
+
+    config = ZIFUNEX_CONFIGS[name][0]
+    plain = Z.PlainZifunex(folders[name])
+    engine = nnis_amd.load_engine(folders[name], dtype=dtype, max_tokens=64 * 9, max_slots=4)
+    yard = Yardstick(plain)
+    for batch_seed, lengths in ((0, [1, 70, 130, 9]), (1, [65, 3, 128]), (2, [2, 2, 200, 64])):
+        requests = [_ids(n + decode, config["vocab"], 100 * batch_seed + i) for i, (n, decode) in enumerate(zip(lengths, (12, 5, 9, 1)))]
+        slots = [engine.start_sequence() for _ in requests]
+        at = list(lengths)
+        logits = engine.step([StepEntry(s, r[:n], list(range(n))) for s, r, n in zip(slots, requests, lengths)]).cpu()
+        row = 0
+        for i, n in enumerate(lengths):
+            yard.check(logits[row:row + n], requests[i], dtype, f"{name} batch {batch_seed} prompt {i}", rows=slice(0, n))
+            row += n
+        live = list(range(len(requests)))
+        while live:
+            live = [i for i in live if at[i] < len(requests[i]) or engine.end_sequence(slots[i])]
+            if not live:
+                break
+            logits = engine.step([StepEntry(slots[i], [requests[i][at[i]]], [0]) for i in live]).cpu()
+            for row, i in enumerate(live):
+                yard.check(logits[row], requests[i], dtype, f"{name} batch {batch_seed} request {i} position {at[i]}", rows=at[i])
+                at[i] += 1
+        assert engine.free_slots() == 4 and engine.free_pages() == 9
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(folders, dtype):
+    config = ZIFUNEX_CONFIGS["B"][0]
+    plain = Z.PlainZifunex(folders["B"])
+    engine = nnis_amd.load_engine(folders["B"], dtype=dtype, max_tokens=512)
+    ids = _ids(330, config["vocab"], 4)
+    slot = engine.start_sequence()
+    got = _collect(engine, slot, ids, [3] + list(range(4, 331)))
+    yard = Yardstick(plain)
+    yard.check(got, ids, dtype, "long decoding")
+    yard.check(got[-1], ids, dtype, "long decoding, the last token", rows=len(ids) - 1)
+
+
+@pytest.mark.parametrize("name", sorted(ZIFUNEX_CONFIGS))
+def test_greedy_generation_through_the_entry_point(folders, name):
+    """``nnis_amd.generate``: the library's scheduler, batches and selection on the device.  In 32-bit the tokens are
+    the plain model's, unless two logits are closer than rounding."""
+    config = ZIFUNEX_CONFIGS[name][0]
+    plain = Z.PlainZifunex(folders[name])
+    prompts = [_ids(n, config["vocab"], 50 + n) for n in (1, 19, 70)]
+    got = nnis_amd.generate(folders[name], prompts, max_new_tokens=10, dtype="float32", stop_token_ids=[])
+    for prompt, tokens in zip(prompts, got):
+        assert len(tokens) == 10
+        logits = plain.logits(prompt + tokens)[len(prompt) - 1:-1]
+        for row, token in zip(logits, tokens):
+            assert float(row[token]) >= float(row.max()) - 1e-4 * float(row.abs().max()), "a generated token is not the plain model's best"
+    got16 = nnis_amd.generate(folders[name], prompts, max_new_tokens=6, dtype="bfloat16", stop_token_ids=[])
+    assert [len(t) for t in got16] == [6, 6, 6]
+
+
+def test_the_command_line_runs_the_model(folders):
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    done = subprocess.run([sys.executable, os.path.join(root, "bin", "nnis"), "generate", "--model", folders["A"], "--prompt-ids", "5,17,3",
+                           "--max-new-tokens", "4", "--dtype", "float32"], capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-2000:]
+    plain = Z.PlainZifunex(folders["A"])
+    assert [int(t) for t in done.stdout.strip().splitlines()[-1].split(",")] == plain.greedy([5, 17, 3], 4)
+
+
+def test_other_sizes_drawn_from_a_seed(tmp_path):
+    """Configurations whose every size is drawn at random, in 32-bit against the plain model: prompt, a portion, single tokens."""
+    import random
+
+    for seed in range(6):
+        r = random.Random(seed)
+        layers = []
+        for _ in range(r.randint(1, 3)):
+            if r.random() < 0.5:
+                dim, vdim = r.choice(HEAD_SIZES)  # (a module is compiled per pair of sizes: those that are built beforehand)
+                layers.append(parallel(attention(r.randint(1, 3) * (k := r.randint(1, 2)), k, dim, vdim, 2 * r.randint(1, dim // 2),
+                                                 base=r.choice([50.0, 1e4, 1e6]), scale=r.uniform(0.05, 0.5), softcap=r.uniform(2.0, 60.0)),
+                                       scan(r.randint(3, 70), r.randint(1, 50), r.randint(1, 9), r.randint(1, 6)),
+                                       ff=r.choice([None, r.randint(8, 90)])))
+            else:
+                layers.append(gla(r.randint(1, 3), r.randint(1, 50), r.randint(1, 50), r.uniform(0.5, 40.0), r.randint(1, 12), ff=r.choice([None, r.randint(8, 90)])))
+        start = r.randint(0, len(layers))
+        config = zifunex(vocab=r.randint(20, 400), width=4 * r.randint(3, 30), streams=r.randint(1, 5), layers=layers,
+                         loop=r.choice([None, (start, r.randint(start, len(layers)), r.randint(1, 3))]), eps=r.choice([1e-5, 1e-6, 1e-3]),
+                         buckets=r.randint(1, 300), mul_prev=r.randint(0, 10 ** 6), mul_cur=r.randint(0, 10 ** 6))
+        folder = str(tmp_path / f"m{seed}")
+        nnis_amd.write_random_model(folder, config, seed)
+        plain = Z.PlainZifunex(folder)
+        engine = nnis_amd.load_engine(folder, dtype="float32", max_tokens=256)
+        ids = _ids(80, config["vocab"], seed)
+        want = plain.logits(ids)
+        slot = engine.start_sequence()
+        got = _collect(engine, slot, ids, [66, 70] + list(range(71, 81)))
+        assert _relative(got, want) < 5e-5, f"seed {seed}: {config}"

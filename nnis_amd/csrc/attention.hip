@@ -40,8 +40,15 @@ constexpr int HD = NNIS_HEAD_DIM;
 #define NNIS_VALUE_DIM NNIS_HEAD_DIM
 #endif
 constexpr int HDV = NNIS_VALUE_DIM;
-// the matrix-core kernels below take heads in steps of 16 channels whose values are as wide as their keys
-#define NNIS_MATRIX_CORES (NNIS_HEAD_DIM % 16 == 0 && NNIS_VALUE_DIM == NNIS_HEAD_DIM)
+// the matrix-core kernels below take heads whose keys and values come in steps of 16 channels
+#define NNIS_MATRIX_CORES (NNIS_HEAD_DIM % 16 == 0 && NNIS_VALUE_DIM % 16 == 0)
+// what a wave's registers are sized by: the larger of the two
+#define NNIS_REG_DIM (NNIS_HEAD_DIM > NNIS_VALUE_DIM ? NNIS_HEAD_DIM : NNIS_VALUE_DIM)
+constexpr int HDR = NNIS_REG_DIM;
+// 1: scores are bent by a cap before the softmax, s -> cap * tanh(s / cap) (compiled in: the kernels of plain scores stay as they are)
+#ifndef NNIS_SCORE_CAP
+#define NNIS_SCORE_CAP 0
+#endif
 
 struct AttnArgs {
   const void* q;  // [tokens, heads, HD]
@@ -163,19 +170,35 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kFullD = HD / 32;       // steps of 32 channels in a score
 constexpr bool kTailD = (HD % 32) != 0;  // plus one of 16
-constexpr int kTilesD = HD / 16;      // output tiles of 16 channels
+constexpr int kTilesD = HDV / 16;     // output tiles of 16 value channels
 // waves of a block: beyond 64 channels a wave needs more registers than a block of 8 waves leaves it
-constexpr int kBlockWaves = HD <= 64 ? 8 : 4;
-constexpr int kPartial = HD + 4;  // floats a split leaves per (token, head), rows 16-byte aligned
+constexpr int kBlockWaves = HDR <= 64 ? 8 : 4;
+constexpr int kPartial = HDV + 4;  // floats a split leaves per (token, head), rows 16-byte aligned
 // key blocks a decoding wave has in flight (its registers hold their operands)
-constexpr int kDecodeRing = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
+constexpr int kDecodeRing = HDR <= 64 ? 4 : (HDR <= 128 ? 2 : 1);
 // the kernel with keys on lanes: pages in flight, and how far a score may rise above the softmax's
 // reference (as a power of two) before the reference moves
-constexpr int kKeysRing = HD <= 64 ? 3 : 2;
+constexpr int kKeysRing = HDR <= 64 ? 3 : 2;
 constexpr int kKeysWaves = 4;  // of a block of that kernel: a wave keeps kKeysRing pages in registers
 constexpr int kKeysMaxHD = 128;
 constexpr float kLazyRise = 8.0f;
 constexpr float kLog2e = 1.4426950408889634f;
+
+// The cap of the scores: a raw score s (a sum of products) becomes out * tanh(s * in), in = scale / cap and
+// out = cap * log2(e): the capped score in the softmax's base-2 units, so that the scale behind it is 1.
+// tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1), right at both ends (the power overflows to infinity or falls to zero).
+struct ScoreCap {
+  float in, out;
+};
+__device__ __forceinline__ void bend(f32x4& s, const ScoreCap& cap) {
+#if NNIS_SCORE_CAP
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float power = __builtin_amdgcn_exp2f(s[e] * cap.in * (2.0f * kLog2e));
+    s[e] = cap.out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(power + 1.0f));
+  }
+#endif
+}
 
 struct QFrag {
   bf16x8 full[kFullD > 0 ? kFullD : 1];
@@ -256,13 +279,16 @@ __device__ __forceinline__ void load_block(BlockFrags& f, const bf16_t* k_page, 
 //   lo[c], hi[c]: the column of this lane reads keys lo <= key <= hi
 template <int C>
 __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, int key0,
-                                             const int (&lo)[C], const int (&hi)[C], float scale_log2, int g) {
+                                             const int (&lo)[C], const int (&hi)[C], float scale_log2, const ScoreCap& cap, int g) {
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     f32x4 s[2];
     float block_max = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) s[t] = score_tile(f.keys[t], q[c]);
+    for (int t = 0; t < 2; ++t) {
+      s[t] = score_tile(f.keys[t], q[c]);
+      bend(s[t], cap);
+    }
     // most blocks lie wholly inside what every lane's column reads: then no key needs a look at its index
     if (!__all(key0 >= lo[c] && key0 + 31 <= hi[c])) {
 #pragma unroll
@@ -328,8 +354,10 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
 // instructions, a few vector instructions, and so on.
 template <int C, bool AHEAD, int c>
 __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
-                                                  f32x4 (&s)[2], bf16x8& before, float scale_log2, float (&rise)[C]) {
+                                                  f32x4 (&s)[2], bf16x8& before, float scale_log2, float (&rise)[C], const ScoreCap& cap) {
   constexpr int kScores = 2 * (kFullD + (kTailD ? 1 : 0));
+  bend(s[0], cap);  // (the scores come in as the matrix unit left them)
+  bend(s[1], cap);
   // rise[c]: the raw score (before the scale) above which column c's reference moves, (st.m[c] + kLazyRise) / scale:
   // the test of every unit is then the scores' maximum against a register
   float block_max = -INFINITY;
@@ -402,14 +430,14 @@ __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag 
     s[0] = ahead[0];
     s[1] = ahead[1];
   }
-  if constexpr (c + 1 < C) attend_unit_ahead<C, AHEAD, c + 1>(st, q, f, next, s, before, scale_log2, rise);
+  if constexpr (c + 1 < C) attend_unit_ahead<C, AHEAD, c + 1>(st, q, f, next, s, before, scale_log2, rise, cap);
 }
 
 template <int C, bool AHEAD>
 __device__ __forceinline__ void attend_block_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
-                                                   f32x4 (&s)[2], float scale_log2, float (&rise)[C]) {
+                                                   f32x4 (&s)[2], float scale_log2, float (&rise)[C], const ScoreCap& cap) {
   bf16x8 before;  // the probabilities of the column before, whose outputs are still to be multiplied
-  attend_unit_ahead<C, AHEAD, 0>(st, q, f, next, s, before, scale_log2, rise);
+  attend_unit_ahead<C, AHEAD, 0>(st, q, f, next, s, before, scale_log2, rise, cap);
 }
 
 // The pages of a run of key blocks, 64 at a time in the lanes of the wave: a
@@ -429,7 +457,7 @@ struct PageRun {
 
 struct MfmaArgs {
   const bf16_t* q;  // [tokens, heads, HD]
-  bf16_t* out;      // [tokens, heads, HD]
+  bf16_t* out;      // [tokens, heads, HDV]
   const bf16_t* k_pages;
   const bf16_t* v_pages;
   const int* block_table;
@@ -438,6 +466,7 @@ struct MfmaArgs {
   int heads, kv_heads;
   int window;
   float scale_log2;
+  ScoreCap cap;  // with NNIS_SCORE_CAP (then scale_log2 is 1)
   // prefill: one work item per (sequence, tile of 16*QT query rows)
   const int* tile_seq;    // [tiles] sequence of the tile
   const int* tile_row0;   // [tiles] first row of the tile within its sequence's new tokens
@@ -455,7 +484,7 @@ __device__ __forceinline__ const bf16_t* k_page_ptr(const MfmaArgs& a, int page,
   return a.k_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(HD);
 }
 __device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page, int kv_head) {
-  return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
+  return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HDV);
 }
 
 // A wave's state in LDS, for another wave to take in: per column the output tiles as 16 bytes a lane
@@ -557,7 +586,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   const int r = lane % 16, g = lane / 16;
   const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
   const bf16_t* v_base = v_page_ptr(a, 0, kv_head);
-  const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HD);
+  const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HDV);
   PageRun run = {pages, a.max_pages, first, stride, 0};
   run.fill(lane);
   // block b of the run: page index first + (b / 2) * stride, half b % 2
@@ -575,7 +604,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
     load_block(into, k_base + page * k_page_stride, v_base + page * v_page_stride, b & 1, r, g);
   };
   auto work = [&](const BlockFrags& f, int b) {
-    attend_block<C>(st, q, f, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
+    attend_block<C>(st, q, f, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, a.cap, g);
   };
   int b0 = 0;
   if (blocks >= 2 * RING) {
@@ -636,7 +665,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 #pragma unroll
           for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[i].keys[t], q[0]);
         }
-        attend_block_ahead<C, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, a.scale_log2, rise);
+        attend_block_ahead<C, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, a.scale_log2, rise, a.cap);
         ask(ring[i], b0 + i + RING);
       }
     }
@@ -660,7 +689,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 // tokens 833 -> 687 us a layer, 24/8 heads of 112 922 -> 652; at 80 and 96 channels, where two waves fit either
 // way, the second block in flight is worth 5 to 8%).
 template <int C>
-constexpr int kPrefillRing = HD > 96 ? (C <= 1 ? 2 : 1) : (HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : NNIS_PREFILL_RING_WIDE));
+constexpr int kPrefillRing = HDR > 96 ? (C <= 1 ? 2 : 1) : (HDR > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : NNIS_PREFILL_RING_WIDE));
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 // An item is a (tile, kv head, chunk of heads); the tiles come longest first, and item i = tile i / per_tile.
@@ -749,7 +778,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
         total += __shfl_xor(total, 32, kWave);
         if (!live[c]) continue;
         const float inv = 1.0f / total;
-        bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HD;
+        bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HDV;
 #pragma unroll
         for (int t = 0; t < kTilesD; ++t) {
           bf16x4 packed;
@@ -812,7 +841,7 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
     for (int c = 0; c < C; ++c) {
       if (!live[c]) continue;
       const float inv = 1.0f / total[c];
-      bf16_t* dst = a.out + ((size_t)token * a.heads + kv_head * group + 16 * c + r) * HD;
+      bf16_t* dst = a.out + ((size_t)token * a.heads + kv_head * group + 16 * c + r) * HDV;
 #pragma unroll
       for (int t = 0; t < kTilesD; ++t) {
         bf16x4 packed;
@@ -830,8 +859,8 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
 #pragma unroll
     for (int t = 0; t < kTilesD; ++t) *(f32x4*)(dst + 16 * t + 4 * g) = st.o[c][t];
     if (g == 0) {
-      dst[HD] = st.m[c];
-      dst[HD + 1] = total[c];
+      dst[HDV] = st.m[c];
+      dst[HDV + 1] = total[c];
     }
   }
 }
@@ -893,7 +922,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(Mfma
 // softmax, which moves only when a score rises more than kLazyRise above it (then every lane's
 // sums are scaled, as in the running maximum; until then they are sums of 2^(score - reference) with
 // terms up to 2^kLazyRise, which changes no result beyond rounding).
-#if NNIS_HEAD_DIM <= 128
+#if NNIS_REG_DIM <= 128
 struct KeysPage {
   bf16x8 k[HD / 8];        // this lane's key, all channels
   bf16x8 v[2][kTilesD];    // value operands of the two halves of the page
@@ -956,7 +985,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
   if (mine > 0) {
     const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
     const bf16_t* v_base = v_page_ptr(a, 0, kv_head);
-    const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HD);
+    const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HDV);
     PageRun run = {pages, a.max_pages, first, stride, 0};
     run.fill(lane);
     KeysPage ring[kKeysRing];
@@ -980,6 +1009,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
         s1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(high4(f.k[c]), high4(q[c]), s1, 0, 0, 0);
       }
       f32x4 s = s0 + s1;
+      bend(s, a.cap);
       const bool inside = key0 >= first_key && key0 + kPageTokens - 1 <= pos;  // every key of the page is read
       float top = -INFINITY;
 #pragma unroll
@@ -1067,7 +1097,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
   }
   finish_decode<1>(st, live, a, merge, token, kv_head, split, wave, waves, lane);
 }
-#endif  // NNIS_HEAD_DIM <= 128
+#endif  // NNIS_REG_DIM <= 128
 
 // sums the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
 // A kernel of its own: letting the last block of a (token, kv head) do it needs a device-wide fence in
@@ -1081,13 +1111,13 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
     // a padding row's runs hold whatever the scratch held: they are read like any (the slot is asked for in the
     // same round trip, not before it) and nothing is stored for them
     const int slot = tok_slot[token];
-    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    for (int d = threadIdx.x; d < HDV; d += blockDim.x) {
       float m[kAtOnce], l[kAtOnce], o[kAtOnce];
 #pragma unroll
       for (int s = 0; s < kAtOnce; ++s) {
         const float* p = base + (size_t)(s < splits ? s : splits - 1) * kPartial;  // (beyond the last: the last again, not counted)
-        m[s] = p[HD];
-        l[s] = p[HD + 1];
+        m[s] = p[HDV];
+        l[s] = p[HDV + 1];
         o[s] = p[d];
       }
       float m_all = -INFINITY;
@@ -1102,23 +1132,23 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
           den += l[s] * w;
         }
       }
-      if (slot >= 0) out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
+      if (slot >= 0) out[((size_t)token * heads + head) * HDV + d] = (bf16_t)(num / den);
     }
     return;
   }
   if (tok_slot[token] < 0) return;
   float m_all = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * kPartial + HD]);
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * kPartial + HDV]);
+  for (int d = threadIdx.x; d < HDV; d += blockDim.x) {
     float num = 0.0f, den = 0.0f;
     for (int s = 0; s < splits; ++s) {
       const float* p = base + (size_t)s * kPartial;
-      const float m = p[HD];
+      const float m = p[HDV];
       const float w = m == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m - m_all);
       num += p[d] * w;
-      den += p[HD + 1] * w;
+      den += p[HDV + 1] * w;
     }
-    out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
+    out[((size_t)token * heads + head) * HDV + d] = (bf16_t)(num / den);
   }
 }
 
@@ -1158,11 +1188,13 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
 
 #if NNIS_MATRIX_CORES
 namespace {
-constexpr int kMaxColumns = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // column tiles a wave carries (registers)
+constexpr int kMaxColumns = HDR <= 64 ? 4 : (HDR <= 128 ? 2 : 1);  // column tiles a wave carries (registers)
 
 int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, const void* v_pages, const int* block_table,
-                int max_pages, int heads, int kv_heads, int head_dim, int window, float scale) {
+                int max_pages, int heads, int kv_heads, int head_dim, int window, float scale, float softcap) {
   NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
+  NNIS_REQUIRE(NNIS_SCORE_CAP ? softcap > 0.0f : softcap == 0.0f,
+               "attention: this module is compiled %s a cap of the scores, got a cap of %g", NNIS_SCORE_CAP ? "with" : "without", (double)softcap);
   NNIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: %d heads do not divide into %d kv heads",
                heads, kv_heads);
   NNIS_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window %d or block table width %d", window, max_pages);
@@ -1172,7 +1204,9 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
                "attention: operands must be 16-byte aligned");
   a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
   a.block_table = block_table; a.max_pages = max_pages; a.heads = heads; a.kv_heads = kv_heads; a.window = window;
-  a.scale_log2 = scale * kLog2e;
+  a.scale_log2 = NNIS_SCORE_CAP ? 1.0f : scale * kLog2e;
+  a.cap.in = NNIS_SCORE_CAP ? scale / softcap : 0.0f;
+  a.cap.out = softcap * kLog2e;
   a.tile_seq = a.tile_row0 = a.seq_slot = a.seq_start = a.seq_pos0 = a.tok_slot = a.tok_pos = nullptr;
   a.splits = 1; a.heads_first = 0; a.partial = nullptr; a.rows_by_token = 0;
   return 0;
@@ -1227,9 +1261,9 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
                                            const int* block_table, int max_pages, const int* tile_seq,
                                            const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
                                            const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
-                                           float scale, int waves, int columns, void* stream) {
+                                           float scale, int waves, int columns, float softcap, void* stream) {
   MfmaArgs a;
-  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
+  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
   if (tiles <= 0) return 0;
   a.tile_seq = tile_seq; a.tile_row0 = tile_row0; a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0;
   const int group = heads / kv_heads;
@@ -1292,7 +1326,7 @@ extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
   const int group = heads / (kv_heads > 0 ? kv_heads : 1);
   const int tiles = (group + 15) / 16;
   const int per_wave = tiles * (kTilesD * 4 + 2) * kWave * 4;  // bytes of LDS a wave's state takes in the merge
-  const int most = (group <= 4 && HD <= kKeysMaxHD && kKeysWaves < kBlockWaves) ? kKeysWaves : kBlockWaves;
+  const int most = (group <= 4 && HDR <= kKeysMaxHD && kKeysWaves < kBlockWaves) ? kKeysWaves : kBlockWaves;
   int waves = 1;
   while (waves * 2 <= most && waves * per_wave <= 65536) waves *= 2;
   return waves;
@@ -1308,9 +1342,9 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
                                           int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
-                                          void* stream) {
+                                          float softcap, void* stream) {
   MfmaArgs a;
-  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
+  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
   a.rows_by_token = rows_by_token ? 1 : 0;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
@@ -1324,7 +1358,7 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   NNIS_REQUIRE(group <= 16 * kMaxColumns, "attention: a group of %d query heads is more than this head size's decode kernel carries (%d)",
                group, 16 * kMaxColumns);
   NNIS_REQUIRE(kind >= 0 && kind <= 2, "attention: unknown decode kernel %d", kind);
-  const bool keys_fit = group <= 4 && HD <= kKeysMaxHD;
+  const bool keys_fit = group <= 4 && HDR <= kKeysMaxHD;
   NNIS_REQUIRE(kind != 2 || keys_fit, "attention: the kernel with keys on lanes takes groups of up to 4 heads of up to %d channels",
                kKeysMaxHD);
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.splits = splits; a.partial = partial;
@@ -1340,13 +1374,13 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   hipStream_t s = (hipStream_t)stream;
   const int tiles = (group + 15) / 16;
   const size_t lds = (size_t)(waves / 2) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
-#if NNIS_HEAD_DIM <= 128
+#if NNIS_REG_DIM <= 128
   {
     if (kind == 2 || (kind == 0 && keys_fit)) {
       hipLaunchKernelGGL(attention_decode_keys_kernel, grid, dim3(kWave * waves), lds, s, a, waves);
       NNIS_LAUNCH_CHECK("attention_decode");
       if (splits > 1 && combine) {
-        hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s,
+        hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HDV < 64 ? 64 : (HDV > 256 ? 256 : HDV)), 0, s,
                            partial, (bf16_t*)out, tok_slot, heads, splits);
         NNIS_LAUNCH_CHECK("attention_combine");
       }
@@ -1359,7 +1393,7 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave * waves), lds, s, a, waves);  // 3 or 4 tiles
   NNIS_LAUNCH_CHECK("attention_decode");
   if (splits > 1 && combine) {
-    hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s, partial,
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HDV < 64 ? 64 : (HDV > 256 ? 256 : HDV)), 0, s, partial,
                        (bf16_t*)out, tok_slot, heads, splits);
     NNIS_LAUNCH_CHECK("attention_combine");
   }
@@ -1370,10 +1404,10 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
 // take the runs as they are.
 extern "C" int nnis_attention_combine(const float* partial, void* out, const int* tok_slot, int tokens, int heads, int head_dim,
                                       int splits, void* stream) {
-  NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
+  NNIS_REQUIRE(head_dim == HDV, "attention: this module is compiled for values of %d channels, got %d", HDV, head_dim);
   NNIS_REQUIRE(partial && out && tok_slot && splits >= 1 && heads > 0, "attention_combine: missing operand");
   if (tokens <= 0) return 0;
-  hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0,
+  hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HDV < 64 ? 64 : (HDV > 256 ? 256 : HDV)), 0,
                      (hipStream_t)stream, partial, (bf16_t*)out, tok_slot, heads, splits);
   NNIS_LAUNCH_CHECK("attention_combine");
   return 0;
@@ -1382,15 +1416,15 @@ extern "C" int nnis_attention_combine(const float* partial, void* out, const int
 extern "C" int nnis_attention_prefill_tile_rows(int, int, int) { return 0; }
 extern "C" int nnis_attention_prefill_max_waves(int, int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                           int, const int*, const int*, const int*, int, int, int, int, float, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+                                           int, const int*, const int*, const int*, int, int, int, int, float, int, int, float, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }
 extern "C" int nnis_attention_combine(const float*, void*, const int*, int, int, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                          int, int, int, int, int, float, int, int, float*, int, int, int, void*) {
-  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16 and values as wide as the keys; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+                                          int, int, int, int, int, float, int, int, float*, int, int, int, float, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 #endif

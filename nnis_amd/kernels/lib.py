@@ -50,7 +50,8 @@ FLAGS = [
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 PREBUILT_HEAD_DIMS = (6, 16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 # values of another size than the keys: what the tests use
-PREBUILT_WIDE_VALUES = ("attn_hd32v16", "attn_hd16v48", "attn_hd48v64", "attn_hd64v32", "attn_hd6v10")
+PREBUILT_WIDE_VALUES = ("attn_hd32v16c", "attn_hd16v48c", "attn_hd48v64c", "attn_hd64v32c", "attn_hd6v10c", "attn_hd32c", "attn_hd64c",
+                        "attn_hd16c", "attn_hd128c", "attn_hd128v64")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -100,9 +101,11 @@ def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], r
 
 
 def _attention_recipe(rest: str) -> ModuleRecipe:
-    """``attn_hd<N>``: keys and values of N channels; ``attn_hd<N>v<M>``: values of M."""
+    """``attn_hd<N>``: keys and values of N channels; ``attn_hd<N>v<M>``: values of M; a ``c`` behind either: with a
+    cap of the scores compiled in."""
+    capped = rest.endswith("c")
     try:
-        sizes = [int(part) for part in rest.split("v")]
+        sizes = [int(part) for part in (rest[:-1] if capped else rest).split("v")]
         if not 1 <= len(sizes) <= 2 or min(sizes) <= 0:
             raise ValueError(rest)
     except ValueError:
@@ -110,6 +113,8 @@ def _attention_recipe(rest: str) -> ModuleRecipe:
     defines = [("NNIS_HEAD_DIM", str(sizes[0]))]
     if len(sizes) == 2:
         defines.append(("NNIS_VALUE_DIM", str(sizes[1])))
+    if capped:
+        defines.append(("NNIS_SCORE_CAP", "1"))
     return ModuleRecipe(("attention.hip",), ("common.h",), tuple(defines), (("attention.hip", tuple(_VECTOR_SUMS)),))
 
 

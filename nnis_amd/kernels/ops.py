@@ -63,10 +63,10 @@ _ATTN_SIGNATURES = {
                             _INT, _INT, _FLT, _INT, _FLT, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
-                                    _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
+                                    _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _VOID],
     "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
-                                   _INT, _INT, _VOID, _INT, _INT, _INT, _VOID],
+                                   _INT, _INT, _VOID, _INT, _INT, _INT, _FLT, _VOID],
     "nnis_attention_combine": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_attention_decode_max_waves": [_INT, _INT],
 }
@@ -158,14 +158,15 @@ def attention_check(head_dim: int, value_dim: Optional[int] = None) -> None:
         raise Unsupported(f"the attention kernels take values of up to {ATTENTION_MOST_CHANNELS} channels, got {value_dim}")
 
 
-def attention_module_name(head_dim: int, value_dim: Optional[int] = None) -> str:
-    """The module compiled for keys of ``head_dim`` channels and values of ``value_dim`` (None: as the keys)."""
+def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0) -> str:
+    """The module compiled for keys of ``head_dim`` channels and values of ``value_dim`` (None: as the keys), with a
+    cap of the scores (``softcap`` > 0) or without."""
     wide = value_dim is not None and value_dim != head_dim
-    return f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}"
+    return (f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}") + ("c" if softcap else "")
 
 
-def attention_module(head_dim: int, value_dim: Optional[int] = None):
-    name = attention_module_name(head_dim, value_dim)
+def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0):
+    name = attention_module_name(head_dim, value_dim, softcap)
     if name not in _attn:
         attention_check(head_dim, value_dim)
         _attn[name] = _bind(name, _ATTN_SIGNATURES)
@@ -448,7 +449,7 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
         raise KernelError("attention: key and value pages differ in type")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
-    lib = attention_module(head_dim, value_dim)
+    lib = attention_module(head_dim, value_dim, softcap)
     _check(lib, lib.nnis_attention_rows(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
                                         v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
                                         tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
@@ -732,11 +733,13 @@ def linear(x: torch.Tensor, weight, out: torch.Tensor) -> torch.Tensor:
     return gemm_ordered(x, weight, out)
 
 
-def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim):
+def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim, value_dim=None):
     tokens = q.shape[0]
-    if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
-        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
-    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
+    value_dim = value_dim or head_dim
+    if q.shape != (tokens, heads * head_dim) or out.shape != (tokens, heads * value_dim):
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim} "
+                          f"with values of {value_dim}")
+    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim, value_dim):
         raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
     if block_table.dtype != torch.int32 or block_table.dim() != 2:
         raise KernelError("attention: block_table must be int32 [slots, pages]")
@@ -746,24 +749,24 @@ def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_di
             raise KernelError(f"attention: the matrix-core kernels take bfloat16, {what} is {t.dtype}")
 
 
-def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0) -> int:
+def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0) -> int:
     """Query rows per work item of ``attention_prefill_bf16`` for these sizes.
     ``columns``: the most 16-column tiles (query tiles x heads of a group) a
     wave carries; 0 for as many as the head size allows."""
-    return attention_module(head_dim).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
+    return attention_module(head_dim, value_dim, softcap).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
 
 
-def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0) -> int:
-    return attention_module(head_dim).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
+def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0) -> int:
+    return attention_module(head_dim, value_dim, softcap).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
 
 
 def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
-                           heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0):
+                           heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0, value_dim=None, softcap=0.0):
     """Causal attention of whole runs of new tokens over the cache, on the
     matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
     sequence of the step and the first of ``prefill_tile_rows`` rows of its
     new tokens; ``seq_start`` [batch + 1] gives each sequence's packed rows."""
-    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
+    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim, value_dim)
     for t in (tile_seq, tile_row0, seq_slot, seq_start, seq_pos0):
         _dev(t, "step metadata")
         if t.dtype != torch.int32:
@@ -771,17 +774,18 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
     tiles = tile_seq.numel()
     if tile_row0.numel() != tiles or seq_start.numel() != seq_slot.numel() + 1 or seq_pos0.numel() != seq_slot.numel():
         raise KernelError("attention: step metadata arrays do not fit each other")
-    lib = attention_module(head_dim)
+    lib = attention_module(head_dim, value_dim, softcap)
     _check(lib, lib.nnis_attention_prefill_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
                                                 block_table.data_ptr(), block_table.shape[1], tile_seq.data_ptr(),
                                                 tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(),
                                                 seq_pos0.data_ptr(), heads, kv_heads, head_dim, int(window), float(scale),
-                                                int(waves), int(columns), _stream()))
+                                                int(waves), int(columns), float(softcap), _stream()))
     return out
 
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
-                          window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False, token_pages=None):
+                          window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False, token_pages=None,
+                          value_dim=None, softcap=0.0):
     """One query token per sequence over its cached keys.  The keys are cut
     into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
@@ -795,7 +799,8 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
     carries) or "auto", which takes "keys" where it fits.  ``token_pages``
     (int32 [tokens, pages], ``StepTables.pages``): each token's sequence's
     pages, read in place of the block table's row of the token's slot."""
-    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
+    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim, value_dim)
+    value_dim = value_dim or head_dim
     tokens = q.shape[0]
     table = block_table
     if token_pages is not None:
@@ -808,18 +813,18 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
         if t.dtype != torch.int32 or t.numel() < tokens:
             raise KernelError("attention: tok_slot / tok_pos must be int32 with one entry per token")
     if splits > 1:
-        if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (head_dim + 4):
-            raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (head_dim + 4)")
+        if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (value_dim + 4):
+            raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (value channels + 4)")
         _dev(partial, "partial")
-    lib = attention_module(head_dim)
+    lib = attention_module(head_dim, value_dim, softcap)
     _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
                                                table.data_ptr(), table.shape[1], tok_slot.data_ptr(),
                                                tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
                                                float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
                                                _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1,
-                                               1 if token_pages is not None else 0, _stream()))
+                                               1 if token_pages is not None else 0, float(softcap), _stream()))
     if keep_runs and splits > 1:
-        return KeyRuns(partial, int(splits), tokens, heads, head_dim, tok_slot, out)
+        return KeyRuns(partial, int(splits), tokens, heads, value_dim, tok_slot, out, lib)
     return out
 
 
@@ -837,9 +842,10 @@ class KeyRuns:
 
     dtype = torch.bfloat16
 
-    def __init__(self, partial, runs, tokens, heads, head_dim, tok_slot, out):
+    def __init__(self, partial, runs, tokens, heads, head_dim, tok_slot, out, module=None):
+        """``head_dim``: the channels of a head's output (its values'); ``module``: the attention module that left the runs."""
         self.partial, self.runs, self.tokens, self.heads, self.head_dim = partial, runs, tokens, heads, head_dim
-        self.tok_slot, self.out = tok_slot, out
+        self.tok_slot, self.out, self.module = tok_slot, out, module
         self.shape = (tokens, heads * head_dim)
 
     def fits(self, rows_out: int) -> bool:
@@ -848,7 +854,7 @@ class KeyRuns:
 
     def combine(self) -> torch.Tensor:
         """The attention's output, added up by the kernel of its own."""
-        lib = attention_module(self.head_dim)
+        lib = self.module or attention_module(self.head_dim)
         _check(lib, lib.nnis_attention_combine(self.partial.data_ptr(), self.out.data_ptr(), self.tok_slot.data_ptr(), self.tokens,
                                                self.heads, self.head_dim, self.runs, _stream()))
         return self.out
@@ -882,8 +888,8 @@ def decode_scratch_held(device):
     return _decode_scratch.get((device.type, device.index))
 
 
-def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
-    return attention_module(head_dim).nnis_attention_decode_max_waves(heads, kv_heads)
+def decode_max_waves(heads: int, kv_heads: int, head_dim: int, value_dim=None, softcap=0.0) -> int:
+    return attention_module(head_dim, value_dim, softcap).nnis_attention_decode_max_waves(heads, kv_heads)
 
 
 def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, width: int = 0):
@@ -1049,26 +1055,27 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     functions choose for the step's planned sizes."""
     value_dim = value_dim or head_dim
     fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap)
-    if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
-        splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * head_dim)
-        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
+    size = max(head_dim, value_dim)  # what a wave's registers are sized by
+    if fast and ctx.decode and heads // kv_heads <= 16 * (4 if size <= 64 else (2 if size <= 128 else 1)):
+        splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * value_dim)
+        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim, value_dim, softcap))
         partial = None
         if splits > 1:
-            partial = decode_scratch(q.device, q.shape[0] * heads * splits * (head_dim + 4))
+            partial = decode_scratch(q.device, q.shape[0] * heads * splits * (value_dim + 4))
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                                      kv_heads, head_dim, scale, window, splits, partial, waves,
                                      keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS,
-                                     token_pages=tables.pages if tables is not None else None)
+                                     token_pages=tables.pages if tables is not None else None, value_dim=value_dim, softcap=softcap)
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
-        waves, columns = plan or prefill_plan(ctx.planned_len, ctx.planned_rows, heads, head_dim, kv_heads)
-        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns))
-        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns)
+        waves, columns = plan or prefill_plan(ctx.planned_len, ctx.planned_rows, heads, size, kv_heads)
+        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns, value_dim, softcap))
+        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns, value_dim, softcap)
         tiles = ctx.lists.device_list(("attention_tiles", rows), lambda new, first, padded: prefill_tile_list(new, first, padded, rows))
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tiles[0], tiles[1],
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
-                                      waves, columns)
+                                      waves, columns, value_dim, softcap)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window, value_dim, softcap)
 
@@ -1076,7 +1083,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
 def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0) -> bool:
     """Whether ``attention`` takes the matrix-core kernels for these types and sizes (else the 32-bit row kernel)."""
     return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
-            and (value_dim or head_dim) == head_dim and not softcap)
+            and (value_dim or head_dim) % 16 == 0)
 
 
 def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, rng: torch.Tensor,

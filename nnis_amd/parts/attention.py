@@ -104,13 +104,13 @@ class CausalSelfAttention(Mixer):
         # (runs of the keys, waves of a block) of a step of single tokens with these sizes
         if not self._matrix_cores(rt):
             return None
-        return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.head_dim)
+        return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.value_dim)
 
     def prompt_plan(self, batch, rows, longest, rt):
         # (waves of a block, columns a wave carries) of the matrix-core kernel; the 32-bit kernel has no plan
         if not self._matrix_cores(rt):
             return None
-        return rt.ops.prefill_plan(longest, rows, self.heads, self.head_dim, self.kv_heads)
+        return rt.ops.prefill_plan(longest, rows, self.heads, max(self.head_dim, self.value_dim), self.kv_heads)
 
     def held_buffers(self, rt):
         # the runs of a decode step's keys meet in a scratch that the kernels' wrapper keeps per device

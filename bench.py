@@ -28,6 +28,12 @@ median of three windows of K steps, one after the other on the same batch; a
 prefill figure is the median of seven runs of a shape seen before.
 ``--workload tinyllama-ragged`` runs that workload alone.
 
+``--workload zifunex`` measures the Zifunex design (attention and a selective
+scan side by side, gated linear attention, several residual streams) at two
+sets of layer sizes of a real model's kind, each beside a Llama of the same
+width, layers, heads, inner size and vocabulary: a prompt of 2,048 tokens in
+one step and decode at batch 1, 8 and 64, all in one JSON line.
+
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
 matrix rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
 """
@@ -63,14 +69,16 @@ def step_flops(config, tokens_per_sequence, wanted_rows):
 class Shape:
     """One model shape with random weights, loaded once; engines of any cache size share its weights."""
 
-    def __init__(self, name, layers, dtype, seed, folder):
+    def __init__(self, name, layers, dtype, seed, folder, config=None, context=None):
+        """``config``: a config.json of any registered architecture instead of the preset ``name``; ``context``: how
+        long its sequences may get here, where the configuration names no last position."""
         import nnis_amd
         from nnis_amd.api import load_model
         from nnis_amd.config import preset
 
         self.name = name
-        self.config = preset(name)
-        self.layers_of_model = self.config["num_hidden_layers"]
+        self.config = preset(name) if config is None else config
+        self.layers_of_model = self.config.get("num_hidden_layers")
         if layers:
             self.config["num_hidden_layers"] = layers
         self.dtype = dtype
@@ -79,8 +87,8 @@ class Shape:
         self.model, self.rt = load_model(folder, dtype=dtype)
         self.load_seconds = time.perf_counter() - started
         self.folder = folder
-        self.context = self.config["max_position_embeddings"]
-        self.vocab = self.config["vocab_size"]
+        self.context = context or self.config["max_position_embeddings"]
+        self.vocab = self.model.spec.vocab_size
 
     def engine(self, max_tokens, max_slots=None):
         from nnis_amd.engine.step import Engine
@@ -207,7 +215,7 @@ def prefill_run(shape, rng, tokens=2048):
     del engine
     torch.cuda.empty_cache()
     seconds = sorted(times[3:])[3]  # the median of seven runs of a shape that has come before (and is captured, where it is)
-    flops = step_flops(shape.config, [tokens], 1)
+    flops = (zifunex_step_flops if shape.config.get("architecture") == "Zifunex" else step_flops)(shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
 
@@ -247,6 +255,87 @@ def ragged_run(shape, rng, sequences=64, shortest=16, longest=1024):
     }
 
 
+# Zifunex at layer sizes of a real model's kind.  Per set: width, inner size of the feed-forwards, (query heads, key/value
+# heads, key channels, value channels) of the attention, (channels, states, rank of the step sizes, taps) of the scan,
+# (heads, key channels, value channels, rank of the decays) of the gated linear attention, streams.  Eight layers: two
+# of attention and scan side by side for one of gated linear attention (which has no feed-forward), twice, then two more.
+ZIFUNEX_SETS = {
+    "w1024": dict(width=1024, ff=2816, attention=(16, 4, 64, 64), scan=(2048, 16, 64, 4), gla=(4, 128, 256, 32), streams=2),
+    "w2048": dict(width=2048, ff=5632, attention=(16, 4, 128, 64), scan=(4096, 16, 128, 4), gla=(8, 128, 256, 32), streams=2),
+}
+ZIFUNEX_LAYERS = "PPGPPGPP"
+ZIFUNEX_VOCAB = 32000
+ZIFUNEX_CONTEXT = 8192  # how far a sequence of these measurements may grow (the design names no last position)
+
+
+def zifunex_config(sizes):
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    inner, states, dt_rank, taps = sizes["scan"]
+    g_heads, g_dim, g_vdim, g_rank = sizes["gla"]
+    side_by_side = {"type": "parallel", "mlp": {"kind": "dense", "ff": sizes["ff"]}, "mixer": {
+        "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot": {"dims": dim, "base": 10000.0},
+                 "scale": dim ** -0.5, "softcap": 30.0},
+        "right": {"inner": inner, "state": states, "dt_rank": dt_rank, "conv": taps}}}
+    linear = {"type": "gla", "mlp": None, "mixer": {"heads": g_heads, "dim": g_dim, "vdim": g_vdim, "tau": 16.0, "rank": g_rank}}
+    return {"architecture": "Zifunex", "vocab": ZIFUNEX_VOCAB, "width": sizes["width"], "streams": sizes["streams"], "norm": {"eps": 1e-5},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+            "layers": [side_by_side if kind == "P" else linear for kind in ZIFUNEX_LAYERS]}
+
+
+def llama_twin_config(sizes):
+    """The closest model the library had: a Llama of the same width, layers, inner size and vocabulary, its heads those
+    of the attention with the value's channels (so that the attention's outputs are as wide)."""
+    from nnis_amd.config import preset
+
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    return preset("tinyllama-1.1b", num_hidden_layers=len(ZIFUNEX_LAYERS), hidden_size=sizes["width"], num_attention_heads=heads,
+                  num_key_value_heads=kv_heads, head_dim=max(dim, vdim), intermediate_size=sizes["ff"], vocab_size=ZIFUNEX_VOCAB,
+                  max_position_embeddings=ZIFUNEX_CONTEXT, tie_word_embeddings=False)
+
+
+def zifunex_step_flops(config, tokens_per_sequence, wanted_rows):
+    """Multiply-adds x2 of one step over whole prompts from empty slots (projections, attention, the two recurrences)."""
+    w = config["width"]
+    total = 0
+    for n in tokens_per_sequence:
+        for layer in config["layers"]:
+            if layer["type"] == "parallel":
+                a, r = layer["mixer"]["left"], layer["mixer"]["right"]
+                per_token = ((a["heads"] + a["kv_heads"]) * a["dim"] + a["kv_heads"] * a["vdim"]) * w + a["heads"] * a["vdim"] * w
+                per_token += 2 * r["inner"] * w + (r["dt_rank"] + 2 * r["state"]) * r["inner"] + r["dt_rank"] * r["inner"] + r["inner"] * w
+                per_token += 3 * r["inner"] * r["state"] + r["conv"] * r["inner"]
+                total += 2 * per_token * n + 2 * a["heads"] * (a["dim"] + a["vdim"]) * n * (n + 1) // 2
+            else:
+                g = layer["mixer"]
+                hd, he = g["heads"] * g["dim"], g["heads"] * g["vdim"]
+                per_token = (2 * hd + 2 * he) * w + g["rank"] * (w + hd) + he * w + 2 * g["heads"] * g["dim"] * g["vdim"]
+                total += 2 * per_token * n
+            if layer["mlp"] is not None:
+                total += 2 * 3 * w * layer["mlp"]["ff"] * n
+    return total + 2 * wanted_rows * w * config["vocab"]
+
+
+def zifunex_run(args, rng):
+    """Each set of sizes: the Zifunex model and its Llama twin, a prompt of 2,048 tokens and decode at batch 1, 8, 64."""
+    import torch
+
+    out = {}
+    for name, sizes in ZIFUNEX_SETS.items():
+        for which, config in (("zifunex", zifunex_config(sizes)), ("llama", llama_twin_config(sizes))):
+            torch.cuda.empty_cache()
+            with tempfile.TemporaryDirectory() as folder:
+                shape = Shape(f"{which}-{name}", 0, args.dtype, args.seed, folder, config=config, context=ZIFUNEX_CONTEXT)
+                record = {"prefill_2048": prefill_run(shape, rng)}
+                for batch in (1, 8, 64):
+                    run = decode_run(shape, rng, batch, args.steps, args.warmup, args.prompt_min, args.prompt_max, windows=3)
+                    record[f"decode_b{batch}"] = {"tokens_per_second": round(run["tokens_per_second"], 1), "ms_per_step": round(run["ms_per_step"], 4),
+                                                  "hbm_frac": round(run["gbs"] / HBM_PEAK_GBS, 4)}
+                record["step_weight_mb"] = round(shape.model.step_weight_bytes() / 1e6, 1)
+                out[f"{which}-{name}"] = record
+                del shape
+    return out
+
+
 def environment():
     import torch
 
@@ -278,7 +367,7 @@ def main() -> int:
     parser.add_argument("--no-other-shapes", action="store_true", help="points of the headline's shape only")
     parser.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     parser.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches (within the context)")
-    parser.add_argument("--workload", choices=["tinyllama-ragged"], help="run this workload alone")
+    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex"], help="run this workload alone")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -287,6 +376,18 @@ def main() -> int:
     import numpy as np
 
     rng = np.random.default_rng(args.seed)
+    if args.workload == "zifunex":
+        models = zifunex_run(args, rng)
+        head = models["zifunex-w2048"]["decode_b8"]
+        print(json.dumps({
+            "metric": "Zifunex at two sets of layer sizes beside a Llama of the same sizes: prefill of 2,048 tokens, decode at batch 1, 8, 64",
+            "value": head["tokens_per_second"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights from a seed, uniform-random token ids",
+            "config": {"model": "Zifunex, 8 layers of width 2048 (decode at batch 8)", "sets": ZIFUNEX_SETS, "layers": ZIFUNEX_LAYERS,
+                       "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
+            "models": models, "env": environment()}))
+        return 0
     with tempfile.TemporaryDirectory() as folder:
         if args.workload == "tinyllama-ragged":
             shape = Shape("tinyllama-1.1b", args.layers, args.dtype, args.seed, folder)

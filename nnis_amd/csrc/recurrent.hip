@@ -122,15 +122,32 @@ struct ScanArgs {
   int channels, states;
   void* y;  // [tokens, channels]
   int y_dtype;
+  // a long run is cut into pieces of `piece` tokens that run side by side (see below)
+  int piece, pieces;
+  float* carried;   // [batch, pieces, channels, states]
+  float* stepped;   // [batch, pieces, channels]: a piece's sum of step sizes
 };
 
-template <int LANES>
+// A run of many tokens is a chain as long as the run.  The recurrence is linear in the state, so the run is cut
+// into pieces that are taken side by side, in three passes: (1) every piece but the last runs from a zero state and
+// leaves what it ends with, E_k, and the sum of its step sizes (the product of its decays is exp(A * that sum));
+// (2) one thread a (channel, state) walks the pieces, I_0 = the sequence's state, I_(k+1) = exp(A sum_k) I_k + E_k,
+// and leaves I_k in E_k's place; (3) every piece runs again, from I_k, and writes the outputs; the last one leaves
+// the sequence's state.  PASS 0 is the plain run of a whole sequence by one block (single tokens, short runs).
+template <int LANES, int PASS>
 __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
-  const int b = blockIdx.y;
+  const int b = blockIdx.z, piece = blockIdx.y;
   const int slot = a.seq_slot[b];
   if (slot < 0) return;
-  const int first = a.seq_start[b], last = a.seq_start[b + 1];
-  if (last <= first) return;
+  const int begin = a.seq_start[b], end = a.seq_start[b + 1];
+  if (end <= begin) return;
+  int first = begin, last = end, pieces_here = 1;
+  if (PASS != 0) {
+    pieces_here = (end - begin + a.piece - 1) / a.piece;
+    if (piece >= pieces_here || (PASS == 1 && piece == pieces_here - 1)) return;
+    first = begin + piece * a.piece;
+    last = min(end, first + a.piece);
+  }
   const int part = threadIdx.x % LANES;
   const int c = blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
   const bool live = c < a.channels;
@@ -138,41 +155,95 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   const int N = a.states;
   float S[8], A[8];
   float* state = a.state + ((size_t)slot * a.channels + cc) * N;
+  float* carried = PASS == 0 ? nullptr : a.carried + (((size_t)b * a.pieces + piece) * a.channels + cc) * N;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int n = part * 8 + j;
-    S[j] = (live && n < N) ? state[n] : 0.0f;
-    A[j] = (live && n < N) ? a.A[(size_t)cc * N + n] : 0.0f;
+    const bool here = live && n < N;
+    S[j] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[n] : carried[n]);
+    A[j] = here ? a.A[(size_t)cc * N + n] : 0.0f;
   }
   const float D = a.D[cc], dt_bias = a.dt_bias[cc];
+  float steps = 0.0f;
+  // the token after this one is asked for before this one is worked on
+  float x_next = load_as_f32(a.x, a.x_dtype, (size_t)first * a.channels + cc);
+  float dt_next = a.dt_pre[(size_t)first * a.channels + cc];
+  float z_next = PASS == 1 ? 0.0f : load_as_f32(a.z, a.z_dtype, (size_t)first * a.z_stride + cc);
+  float B_next[8], C_next[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int n = part * 8 + j;
+    B_next[j] = n < N ? a.bc[(size_t)first * 2 * N + n] : 0.0f;
+    C_next[j] = (PASS != 1 && n < N) ? a.bc[(size_t)first * 2 * N + N + n] : 0.0f;
+  }
   for (int t = first; t < last; ++t) {
-    const float x = load_as_f32(a.x, a.x_dtype, (size_t)t * a.channels + cc);
-    const float dt = softplus_f(a.dt_pre[(size_t)t * a.channels + cc] + dt_bias);
-    const float* B = a.bc + (size_t)t * 2 * N;
-    const float* C = B + N;
-    const float dx = dt * x;
-    float acc = 0.0f;
+    const float x = x_next, z = z_next;
+    const float dt = softplus_f(dt_next + dt_bias);
+    float B[8], C[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      B[j] = B_next[j];
+      C[j] = C_next[j];
+    }
+    const int ahead = t + 1 < last ? t + 1 : t;
+    x_next = load_as_f32(a.x, a.x_dtype, (size_t)ahead * a.channels + cc);
+    dt_next = a.dt_pre[(size_t)ahead * a.channels + cc];
+    if (PASS != 1) z_next = load_as_f32(a.z, a.z_dtype, (size_t)ahead * a.z_stride + cc);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int n = part * 8 + j;
       if (n < N) {
-        S[j] = fmaf(expf(dt * A[j]), S[j], dx * B[n]);
-        acc = fmaf(S[j], C[n], acc);
+        B_next[j] = a.bc[(size_t)ahead * 2 * N + n];
+        if (PASS != 1) C_next[j] = a.bc[(size_t)ahead * 2 * N + N + n];
       }
     }
-#pragma unroll
-    for (int offset = LANES / 2; offset > 0; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
-    if (part == 0 && live) {
-      const float z = load_as_f32(a.z, a.z_dtype, (size_t)t * a.z_stride + c);
-      store_from_f32(a.y, a.y_dtype, (size_t)t * a.channels + c, (acc + D * x) * (z * sigmoid_f(z)));
-    }
-  }
-  if (live) {
+    const float dx = dt * x;
+    steps += dt;
+    float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int n = part * 8 + j;
-      if (n < N) state[n] = S[j];
+      S[j] = fmaf(expf(dt * A[j]), S[j], dx * B[j]);  // (lanes beyond the states: A, B and S are zero)
+      acc = fmaf(S[j], C[j], acc);
     }
+    if (PASS != 1) {
+#pragma unroll
+      for (int offset = LANES / 2; offset > 0; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
+      if (part == 0 && live) store_from_f32(a.y, a.y_dtype, (size_t)t * a.channels + c, (acc + D * x) * (z * sigmoid_f(z)));
+    }
+  }
+  if (!live) return;
+  if (PASS == 1) {
+    if (part == 0) a.stepped[((size_t)b * a.pieces + piece) * a.channels + c] = steps;
+  } else if (PASS == 3 && piece != pieces_here - 1) {
+    return;
+  }
+  float* into = PASS == 1 ? carried : state;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int n = part * 8 + j;
+    if (n < N) into[n] = S[j];
+  }
+}
+
+// pass (2): a thread a (sequence, channel, state)
+__global__ void selective_scan_carry_kernel(ScanArgs a) {
+  const int b = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot < 0 || i >= a.channels * a.states) return;
+  const int count = a.seq_start[b + 1] - a.seq_start[b];
+  if (count <= 0) return;
+  const int pieces_here = (count + a.piece - 1) / a.piece;
+  const int c = i / a.states;
+  const float A = a.A[i];
+  float I = a.state[(size_t)slot * a.channels * a.states + i];
+  for (int k = 0; k < pieces_here; ++k) {
+    float* at = a.carried + ((size_t)b * a.pieces + k) * a.channels * a.states + i;
+    const bool more = k + 1 < pieces_here;
+    const float E = more ? *at : 0.0f;
+    const float steps = more ? a.stepped[((size_t)b * a.pieces + k) * a.channels + c] : 0.0f;
+    *at = I;
+    I = fmaf(expf(A * steps), I, E);
   }
 }
 
@@ -200,17 +271,30 @@ struct GlaArgs {
   int heads, key_dim, value_dim;
   int chunk;   // tokens staged at a time
   float* out;  // [tokens, heads * value_dim]
+  // a long run is cut into pieces of `piece` tokens that run side by side, as the selective scan's
+  int piece, pieces;
+  float* carried;  // [batch, pieces, heads, key_dim, value_dim]
+  float* decayed;  // [batch, pieces, heads, key_dim]: a piece's sum of the decays' logarithms
 };
 
-template <int GROUPS>
+// PASS as in selective_scan_kernel: 0 a whole run; 1 a piece from a zero state, leaving its end and the sum of its
+// decays' logarithms; 3 a piece from the state that the carry kernel left for it, writing the outputs.
+template <int GROUPS, int PASS>
 __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
   extern __shared__ float lds[];
   constexpr int kCols = 4 * (kWave / GROUPS);  // value columns of a block (4 waves)
-  const int b = blockIdx.z, head = blockIdx.y;
+  const int b = blockIdx.z / a.pieces, piece = blockIdx.z % a.pieces, head = blockIdx.y;
   const int slot = a.seq_slot[b];
   if (slot < 0) return;
-  const int first = a.seq_start[b], last = a.seq_start[b + 1];
-  if (last <= first) return;
+  const int begin = a.seq_start[b], end = a.seq_start[b + 1];
+  if (end <= begin) return;
+  int first = begin, last = end, pieces_here = 1;
+  if (PASS != 0) {
+    pieces_here = (end - begin + a.piece - 1) / a.piece;
+    if (piece >= pieces_here || (PASS == 1 && piece == pieces_here - 1)) return;
+    first = begin + piece * a.piece;
+    last = min(end, first + a.piece);
+  }
   const int d = a.key_dim, e = a.value_dim;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int group = lane / (kWave / GROUPS);
@@ -223,23 +307,29 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
   float* vs = as + a.chunk * d;       // [chunk][kCols]
   float S[16];
   float* state = a.state + (((size_t)slot * a.heads + head) * d) * e + (live ? col : 0);
+  float* carried = PASS == 0 ? nullptr : a.carried + ((((size_t)b * a.pieces + piece) * a.heads + head) * d) * e + (live ? col : 0);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int row = group * 16 + r;
-    S[r] = (live && row < d) ? state[(size_t)row * e] : 0.0f;
+    const bool here = live && row < d;
+    S[r] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[(size_t)row * e] : carried[(size_t)row * e]);
   }
+  float log_sum = 0.0f;  // PASS 1, threads below key_dim of the first slab: the sum of a key channel's log decays
   for (int t0 = first; t0 < last; t0 += a.chunk) {
     const int count = min(a.chunk, last - t0);
     __syncthreads();  // the chunk before has been read
     for (int i = threadIdx.x; i < count * d; i += blockDim.x) {
       const int t = t0 + i / d, ch = i % d;
-      qs[i] = load_as_f32(a.q, a.qkv_dtype, (size_t)t * a.q_stride + head * d + ch) * a.scale;
+      if (PASS != 1) qs[i] = load_as_f32(a.q, a.qkv_dtype, (size_t)t * a.q_stride + head * d + ch) * a.scale;
       ks[i] = load_as_f32(a.k, a.qkv_dtype, (size_t)t * a.k_stride + head * d + ch);
       as[i] = expf(log_sigmoid_f(a.zd[((size_t)t * a.heads + head) * d + ch]) * a.inv_tau);
     }
     for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
       const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
       vs[i] = cl < e ? load_as_f32(a.v, a.qkv_dtype, (size_t)t * a.v_stride + head * e + cl) : 0.0f;
+    }
+    if (PASS == 1 && blockIdx.x == 0 && (int)threadIdx.x < d) {
+      for (int j = 0; j < count; ++j) log_sum += log_sigmoid_f(a.zd[((size_t)(t0 + j) * a.heads + head) * d + threadIdx.x]) * a.inv_tau;
     }
     __syncthreads();
     for (int j = 0; j < count; ++j) {
@@ -252,20 +342,47 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
       for (int r = 0; r < 16; ++r) {
         if (group * 16 + r < d) {
           S[r] = fmaf(aj[r], S[r], kj[r] * v);
-          acc = fmaf(S[r], qj[r], acc);
+          if (PASS != 1) acc = fmaf(S[r], qj[r], acc);
         }
       }
+      if (PASS != 1) {
 #pragma unroll
-      for (int offset = kWave / 2; offset >= kWave / GROUPS; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
-      if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+        for (int offset = kWave / 2; offset >= kWave / GROUPS; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
+        if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+      }
     }
   }
-  if (live) {
+  if (PASS == 1 && blockIdx.x == 0 && (int)threadIdx.x < d)
+    a.decayed[(((size_t)b * a.pieces + piece) * a.heads + head) * d + threadIdx.x] = log_sum;
+  if (!live || (PASS == 3 && piece != pieces_here - 1)) return;
+  float* into = PASS == 1 ? carried : state;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = group * 16 + r;
-      if (row < d) state[(size_t)row * e] = S[r];
-    }
+  for (int r = 0; r < 16; ++r) {
+    const int row = group * 16 + r;
+    if (row < d) into[(size_t)row * e] = S[r];
+  }
+}
+
+// between the passes: a thread an element of a sequence's state walks the pieces, I_(k+1) = P_k I_k + E_k with P_k the
+// product of piece k's decays of the element's key channel, and leaves I_k in E_k's place
+__global__ void gla_carry_kernel(GlaArgs a) {
+  const int b = blockIdx.y;
+  const int slot = a.seq_slot[b];
+  const size_t per = (size_t)a.heads * a.key_dim * a.value_dim;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot < 0 || i >= per) return;
+  const int count = a.seq_start[b + 1] - a.seq_start[b];
+  if (count <= 0) return;
+  const int pieces_here = (count + a.piece - 1) / a.piece;
+  const size_t row = i / a.value_dim;  // (head, key channel)
+  float I = a.state[(size_t)slot * per + i];
+  for (int k = 0; k < pieces_here; ++k) {
+    float* at = a.carried + ((size_t)b * a.pieces + k) * per + i;
+    const bool more = k + 1 < pieces_here;
+    const float E = more ? *at : 0.0f;
+    const float logs = more ? a.decayed[((size_t)b * a.pieces + k) * a.heads * a.key_dim + row] : 0.0f;
+    *at = I;
+    I = fmaf(expf(logs), I, E);
   }
 }
 
@@ -318,46 +435,68 @@ extern "C" int nnis_conv_silu(const void* x, int x_dtype, int x_stride, const vo
   return 0;
 }
 
+// piece, pieces: 0, or a run is cut into up to `pieces` pieces of `piece` tokens (then `carried`, float32 of batch * pieces *
+// channels * states, and `stepped`, of batch * pieces * channels, are scratch of the call)
 extern "C" int nnis_selective_scan(const void* x, int x_dtype, const float* dt_pre, const float* bc, const void* z, int z_dtype,
                                    int z_stride, const float* A, const float* D, const float* dt_bias, float* state,
                                    const int* seq_slot, const int* seq_start, int batch, int channels, int states, void* y,
-                                   int y_dtype, void* stream) {
+                                   int y_dtype, int piece, int pieces, float* carried, float* stepped, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(z_dtype) && nnis_dtype_ok(y_dtype), "selective_scan: unknown dtype");
   NNIS_REQUIRE(channels > 0 && states > 0 && states <= 128 && z_stride >= channels && batch >= 0,
                "selective_scan: bad sizes (channels %d, states %d: up to 128 are taken)", channels, states);
   NNIS_REQUIRE(x && dt_pre && bc && z && A && D && dt_bias && state && seq_slot && seq_start && y, "selective_scan: a pointer is missing");
+  NNIS_REQUIRE(pieces <= 1 || (piece > 0 && carried && stepped && pieces <= 65535), "selective_scan: pieces need their length and scratch");
+  NNIS_REQUIRE(batch <= 65535, "selective_scan: %d sequences exceed the grid limit", batch);
   if (batch == 0) return 0;
   ScanArgs a;
   a.x = x; a.x_dtype = x_dtype; a.dt_pre = dt_pre; a.bc = bc; a.z = z; a.z_dtype = z_dtype; a.z_stride = z_stride; a.A = A; a.D = D;
   a.dt_bias = dt_bias; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.channels = channels; a.states = states;
-  a.y = y; a.y_dtype = y_dtype;
+  a.y = y; a.y_dtype = y_dtype; a.piece = piece; a.pieces = pieces; a.carried = carried; a.stepped = stepped;
   const int need = (states + 7) / 8;
   hipStream_t s = (hipStream_t)stream;
-#define NNIS_SCAN(LANES_)                                                                                                  \
-  hipLaunchKernelGGL(selective_scan_kernel<LANES_>, dim3((channels + 256 / LANES_ - 1) / (256 / LANES_), batch), dim3(256), 0, s, a)
-  if (need <= 1) NNIS_SCAN(1);
-  else if (need <= 2) NNIS_SCAN(2);
-  else if (need <= 4) NNIS_SCAN(4);
-  else if (need <= 8) NNIS_SCAN(8);
-  else NNIS_SCAN(16);
+#define NNIS_SCAN(LANES_, PASS_, PIECES_)                                                                                  \
+  hipLaunchKernelGGL((selective_scan_kernel<LANES_, PASS_>), dim3((channels + 256 / LANES_ - 1) / (256 / LANES_), PIECES_, batch), \
+                     dim3(256), 0, s, a)
+#define NNIS_SCAN_PASS(PASS_, PIECES_)                 \
+  do {                                                 \
+    if (need <= 1) NNIS_SCAN(1, PASS_, PIECES_);       \
+    else if (need <= 2) NNIS_SCAN(2, PASS_, PIECES_);  \
+    else if (need <= 4) NNIS_SCAN(4, PASS_, PIECES_);  \
+    else if (need <= 8) NNIS_SCAN(8, PASS_, PIECES_);  \
+    else NNIS_SCAN(16, PASS_, PIECES_);                \
+  } while (0)
+  if (pieces <= 1) {
+    NNIS_SCAN_PASS(0, 1);
+  } else {
+    NNIS_SCAN_PASS(1, pieces);
+    hipLaunchKernelGGL(selective_scan_carry_kernel, dim3((channels * states + 255) / 256, batch), dim3(256), 0, s, a);
+    NNIS_SCAN_PASS(3, pieces);
+  }
+#undef NNIS_SCAN_PASS
 #undef NNIS_SCAN
   NNIS_LAUNCH_CHECK("selective_scan");
   return 0;
 }
 
+// piece, pieces: as nnis_selective_scan's (`carried`: batch * pieces * heads * key_dim * value_dim floats, `decayed`:
+// batch * pieces * heads * key_dim)
 extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
                              const float* zd, float tau, float scale, float* state, const int* seq_slot, const int* seq_start,
-                             int batch, int heads, int key_dim, int value_dim, float* out, void* stream) {
+                             int batch, int heads, int key_dim, int value_dim, float* out, int piece, int pieces, float* carried,
+                             float* decayed, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype), "gla_scan: unknown dtype %d", qkv_dtype);
   NNIS_REQUIRE(heads > 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
                "gla_scan: bad sizes (heads %d, key channels %d: up to 256 are taken, value channels %d)", heads, key_dim, value_dim);
   NNIS_REQUIRE(tau > 0.0f, "gla_scan: tau must be positive, got %g", (double)tau);
   NNIS_REQUIRE(q && k && v && zd && state && seq_slot && seq_start && out, "gla_scan: a pointer is missing");
+  NNIS_REQUIRE(pieces <= 1 || (piece > 0 && carried && decayed), "gla_scan: pieces need their length and scratch");
+  if (pieces < 1) pieces = 1;
+  NNIS_REQUIRE((long long)batch * pieces <= 65535 && heads <= 65535, "gla_scan: %d sequences x %d pieces exceed the grid limit", batch, pieces);
   if (batch == 0) return 0;
   GlaArgs a;
   a.q = q; a.k = k; a.v = v; a.qkv_dtype = qkv_dtype; a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.zd = zd;
   a.inv_tau = 1.0f / tau; a.scale = scale; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads;
-  a.key_dim = key_dim; a.value_dim = value_dim; a.out = out;
+  a.key_dim = key_dim; a.value_dim = value_dim; a.out = out; a.piece = piece; a.pieces = pieces; a.carried = carried; a.decayed = decayed;
   const int need = (key_dim + 15) / 16;
   const int groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
   const int cols = 4 * (kWave / groups);
@@ -365,15 +504,27 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
   chunk = chunk > 32 ? 32 : (chunk < 1 ? 1 : chunk);
   a.chunk = chunk;
   const size_t lds = (size_t)chunk * (3 * key_dim + cols) * sizeof(float);
-  const dim3 grid((value_dim + cols - 1) / cols, heads, batch);
+  const dim3 grid((value_dim + cols - 1) / cols, heads, batch * pieces);
   hipStream_t s = (hipStream_t)stream;
-  switch (groups) {
-    case 1: hipLaunchKernelGGL(gla_scan_kernel<1>, grid, dim3(256), lds, s, a); break;
-    case 2: hipLaunchKernelGGL(gla_scan_kernel<2>, grid, dim3(256), lds, s, a); break;
-    case 4: hipLaunchKernelGGL(gla_scan_kernel<4>, grid, dim3(256), lds, s, a); break;
-    case 8: hipLaunchKernelGGL(gla_scan_kernel<8>, grid, dim3(256), lds, s, a); break;
-    default: hipLaunchKernelGGL(gla_scan_kernel<16>, grid, dim3(256), lds, s, a); break;
+#define NNIS_GLA(PASS_)                                                                                   \
+  do {                                                                                                    \
+    switch (groups) {                                                                                     \
+      case 1: hipLaunchKernelGGL((gla_scan_kernel<1, PASS_>), grid, dim3(256), lds, s, a); break;         \
+      case 2: hipLaunchKernelGGL((gla_scan_kernel<2, PASS_>), grid, dim3(256), lds, s, a); break;         \
+      case 4: hipLaunchKernelGGL((gla_scan_kernel<4, PASS_>), grid, dim3(256), lds, s, a); break;         \
+      case 8: hipLaunchKernelGGL((gla_scan_kernel<8, PASS_>), grid, dim3(256), lds, s, a); break;         \
+      default: hipLaunchKernelGGL((gla_scan_kernel<16, PASS_>), grid, dim3(256), lds, s, a); break;       \
+    }                                                                                                     \
+  } while (0)
+  if (pieces <= 1) {
+    NNIS_GLA(0);
+  } else {
+    NNIS_GLA(1);
+    const size_t per = (size_t)heads * key_dim * value_dim;
+    hipLaunchKernelGGL(gla_carry_kernel, dim3((unsigned)((per + 255) / 256), batch), dim3(256), 0, s, a);
+    NNIS_GLA(3);
   }
+#undef NNIS_GLA
   NNIS_LAUNCH_CHECK("gla_scan");
   return 0;
 }

@@ -75,9 +75,9 @@ _RECURRENT_SIGNATURES = {
     "nnis_conv_silu": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT,
                        _VOID],
     "nnis_selective_scan": [_VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT,
-                            _VOID, _INT, _VOID],
+                            _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_gla_scan": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT,
-                      _VOID, _VOID],
+                      _VOID, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
 }
 
@@ -1254,6 +1254,26 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
 # mixers that carry state
 # ---------------------------------------------------------------------------
 
+# A run of a sequence's tokens through a recurrence is a chain as long as the run; from RUN_PIECE_FROM tokens on the
+# kernels cut it into pieces that run side by side (three passes, see csrc/recurrent.hip).  A piece has at least
+# RUN_PIECE_LEAST tokens; the pieces' states between the passes take at most RUN_SCRATCH_BYTES.
+RUN_PIECE_FROM = 48
+RUN_PIECE_LEAST = 16
+RUN_SCRATCH_BYTES = 256 << 20
+
+
+def run_pieces(ctx, state_bytes: int):
+    """(tokens of a piece, most pieces of a sequence) for a step whose longest run has ``ctx.max_new`` tokens, where a
+    sequence's state takes ``state_bytes``; (0, 1) for a step that is not cut."""
+    longest = int(ctx.max_new)
+    if longest < RUN_PIECE_FROM:
+        return 0, 1
+    most = max(1, min(64, RUN_SCRATCH_BYTES // max(1, ctx.batch * state_bytes)))
+    piece = max(RUN_PIECE_LEAST, -(-longest // most))
+    pieces = -(-longest // piece)
+    return (piece, pieces) if pieces > 1 else (0, 1)
+
+
 def _step_arrays(ctx, what: str):
     for t in (ctx.tok_slot, ctx.tok_pos, ctx.seq_slot, ctx.seq_start):
         _dev(t, "step metadata")
@@ -1306,11 +1326,16 @@ def selective_scan(x: torch.Tensor, dt_pre: torch.Tensor, bc: torch.Tensor, z: t
     if not z.is_cuda or tuple(z.shape) != (tokens, channels) or z.stride(1) != 1:
         raise KernelError("selective_scan: z must be [tokens, channels] on the GPU with adjacent columns")
     _step_arrays(ctx, "selective_scan")
+    piece, pieces = run_pieces(ctx, channels * states * 4)
+    carried = stepped = None
+    if pieces > 1:
+        carried = torch.empty(ctx.batch * pieces * channels * states, dtype=torch.float32, device=x.device)
+        stepped = torch.empty(ctx.batch * pieces * channels, dtype=torch.float32, device=x.device)
     lib = recurrent()
     _check(lib, lib.nnis_selective_scan(x.data_ptr(), _code(x), dt_pre.data_ptr(), bc.data_ptr(), z.data_ptr(), _code(z),
                                         z.stride(0) if tokens > 1 else channels, A.data_ptr(), D.data_ptr(), dt_bias.data_ptr(),
                                         state.data_ptr(), ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(), ctx.batch, channels,
-                                        states, out.data_ptr(), _code(out), _stream()))
+                                        states, out.data_ptr(), _code(out), piece, pieces, _ptr(carried), _ptr(stepped), _stream()))
     return out
 
 
@@ -1336,10 +1361,16 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logits: to
         raise KernelError("gla_scan: out must be float32 [tokens, heads * value channels]")
     _step_arrays(ctx, "gla_scan")
     stride = lambda t: t.stride(0) if tokens > 1 else t.shape[1]  # noqa: E731
+    piece, pieces = run_pieces(ctx, heads * key_dim * value_dim * 4)
+    carried = decayed = None
+    if pieces > 1:
+        carried = torch.empty(ctx.batch * pieces * heads * key_dim * value_dim, dtype=torch.float32, device=out.device)
+        decayed = torch.empty(ctx.batch * pieces * heads * key_dim, dtype=torch.float32, device=out.device)
     lib = recurrent()
     _check(lib, lib.nnis_gla_scan(q.data_ptr(), k.data_ptr(), v.data_ptr(), _code(q), stride(q), stride(k), stride(v),
                                   decay_logits.data_ptr(), float(tau), float(scale), state.data_ptr(), ctx.seq_slot.data_ptr(),
-                                  ctx.seq_start.data_ptr(), ctx.batch, heads, key_dim, value_dim, out.data_ptr(), _stream()))
+                                  ctx.seq_start.data_ptr(), ctx.batch, heads, key_dim, value_dim, out.data_ptr(), piece, pieces,
+                                  _ptr(carried), _ptr(decayed), _stream()))
     return out
 
 

@@ -14,7 +14,11 @@ extern "C" const char* nnis_last_error() { return g_nnis_error; }
 
 namespace {
 
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+constexpr float kLog2e = 1.4426950408889634f;
+// 2^x by the hardware's instruction (about one unit in the last place): the decays of a recurrence are powers of
+// two of a product that is made once, exp(dt A) = 2^(dt (A log2 e))
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.0f + exp2_fast(-z * kLog2e)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 // log(sigmoid(z)) = min(z, 0) - log(1 + exp(-|z|))
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
@@ -43,33 +47,96 @@ struct ConvArgs {
   int y_dtype;
 };
 
-__global__ void conv_silu_kernel(ConvArgs a) {
-  const size_t total = (size_t)a.tokens * a.channels;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    const int token = (int)(i / a.channels), c = (int)(i % a.channels);
+// the input `back` tokens before row `token` of the sequence in `slot` at position `pos` (back <= pos): a row of
+// this step while the rows belong to the sequence, then the state's rows, newest last
+__device__ __forceinline__ float conv_input(const ConvArgs& a, int token, int slot, int back, int c, bool& in_step, int& behind) {
+  if (in_step && token - back >= 0 && a.tok_slot[token - back] == slot)
+    return load_as_f32(a.x, a.x_dtype, (size_t)(token - back) * a.x_stride + c);
+  in_step = false;
+  ++behind;
+  return a.state[((size_t)slot * (a.taps - 1) + (a.taps - 1 - behind)) * a.channels + c];
+}
+
+// A thread takes one channel over a strip of consecutive rows: its taps stay in registers and so do the last inputs
+// while the rows go on in one sequence (one load a row); at a strip's or a sequence's first row they are looked up.
+constexpr int kConvStrip = 16;
+
+__global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.channels) return;
+  const int begin = blockIdx.y * kConvStrip, end = min(a.tokens, begin + kConvStrip);
+  float w[kMostTaps], held[kMostTaps];  // held[j]: the input taps - 1 - j tokens back
+#pragma unroll
+  for (int j = 0; j < kMostTaps; ++j) {
+    w[j] = j < a.taps ? load_as_f32(a.weight, a.weight_dtype, (size_t)c * a.taps + j) : 0.0f;
+    held[j] = 0.0f;
+  }
+  const float bias = a.bias ? load_as_f32(a.bias, a.weight_dtype, c) : 0.0f;
+  int before = -2;  // the slot of the row before, if its inputs are held
+  for (int token = begin; token < end; ++token) {
     const int slot = a.tok_slot[token];
     if (slot < 0) {
-      store_from_f32(a.y, a.y_dtype, i, 0.0f);
+      store_from_f32(a.y, a.y_dtype, (size_t)token * a.channels + c, 0.0f);
+      before = -2;
       continue;
     }
-    const int pos = a.tok_pos[token];
-    float acc = a.bias ? load_as_f32(a.bias, a.weight_dtype, c) : 0.0f;
-    bool in_step = true;  // the rows token, token - 1, ... while they belong to this sequence
-    int behind = 0;       // how many inputs of the state have been used
-    for (int back = 0; back < a.taps; ++back) {
-      if (back > pos) break;  // before the sequence's start: zeros
-      float v;
-      if (in_step && token - back >= 0 && a.tok_slot[token - back] == slot) {
-        v = load_as_f32(a.x, a.x_dtype, (size_t)(token - back) * a.x_stride + c);
-      } else {
-        in_step = false;
-        ++behind;  // the newest input of the state is its last row
-        v = a.state[((size_t)slot * (a.taps - 1) + (a.taps - 1 - behind)) * a.channels + c];
+    if (slot == before) {
+#pragma unroll
+      for (int j = 0; j + 1 < kMostTaps; ++j)
+        if (j + 1 < a.taps) held[j] = held[j + 1];
+      const float now = load_as_f32(a.x, a.x_dtype, (size_t)token * a.x_stride + c);
+#pragma unroll
+      for (int j = 0; j < kMostTaps; ++j)
+        if (j == a.taps - 1) held[j] = now;
+    } else {
+      const int pos = a.tok_pos[token];
+      bool in_step = true;
+      int behind = 0;
+#pragma unroll
+      for (int back = 0; back < kMostTaps; ++back) {
+        if (back < a.taps) {
+          const float v = back <= pos ? conv_input(a, token, slot, back, c, in_step, behind) : 0.0f;  // zeros before the start
+#pragma unroll
+          for (int j = 0; j < kMostTaps; ++j)
+            if (j == a.taps - 1 - back) held[j] = v;
+        }
       }
-      acc = fmaf(load_as_f32(a.weight, a.weight_dtype, (size_t)c * a.taps + (a.taps - 1 - back)), v, acc);
+      before = slot;
     }
-    store_from_f32(a.y, a.y_dtype, i, acc / (1.0f + expf(-acc)));
+    float acc = bias;
+#pragma unroll
+    for (int j = 0; j < kMostTaps; ++j) acc = fmaf(w[j], held[j], acc);  // (beyond the taps: zeros)
+    store_from_f32(a.y, a.y_dtype, (size_t)token * a.channels + c, acc * sigmoid_f(acc));
   }
+}
+
+// A step of single tokens: output and state in one kernel, a thread a (sequence, channel).  The state's rows
+// before a sequence's start are zeros (a slot starts so, and they are only ever moved down).
+__global__ __launch_bounds__(256) void conv_single_kernel(ConvArgs a) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.channels) return;
+  const int token = a.seq_start[b];
+  const int slot = a.seq_slot[b];
+  if (slot < 0) {
+    store_from_f32(a.y, a.y_dtype, (size_t)token * a.channels + c, 0.0f);
+    return;
+  }
+  const int keep = a.taps - 1;
+  float* state = a.state + (size_t)slot * keep * a.channels + c;
+  const float now = load_as_f32(a.x, a.x_dtype, (size_t)token * a.x_stride + c);
+  float acc = a.bias ? load_as_f32(a.bias, a.weight_dtype, c) : 0.0f;
+  float older[kMostTaps];
+#pragma unroll
+  for (int j = 0; j < kMostTaps; ++j) {
+    older[j] = j < keep ? state[(size_t)j * a.channels] : 0.0f;
+    if (j < keep) acc = fmaf(load_as_f32(a.weight, a.weight_dtype, (size_t)c * a.taps + j), older[j], acc);
+  }
+  acc = fmaf(load_as_f32(a.weight, a.weight_dtype, (size_t)c * a.taps + keep), now, acc);
+  store_from_f32(a.y, a.y_dtype, (size_t)token * a.channels + c, acc * sigmoid_f(acc));
+#pragma unroll
+  for (int j = 0; j < kMostTaps; ++j)
+    if (j < keep) state[(size_t)j * a.channels] = j + 1 < keep ? older[j + 1] : now;
 }
 
 // after the outputs are taken: the state becomes the last taps - 1 inputs of each sequence (one thread a
@@ -161,7 +228,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
     const int n = part * 8 + j;
     const bool here = live && n < N;
     S[j] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[n] : carried[n]);
-    A[j] = here ? a.A[(size_t)cc * N + n] : 0.0f;
+    A[j] = here ? a.A[(size_t)cc * N + n] * kLog2e : 0.0f;  // (in powers of two)
   }
   const float D = a.D[cc], dt_bias = a.dt_bias[cc];
   float steps = 0.0f;
@@ -178,7 +245,9 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   }
   for (int t = first; t < last; ++t) {
     const float x = x_next, z = z_next;
-    const float dt = softplus_f(dt_next + dt_bias);
+    // (the step size is the same in all lanes of a channel: one of them takes the logarithm)
+    float dt = part == 0 ? softplus_f(dt_next + dt_bias) : 0.0f;
+    if (LANES > 1) dt = __shfl(dt, (threadIdx.x % kWave) & ~(LANES - 1), kWave);
     float B[8], C[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -202,7 +271,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
     float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      S[j] = fmaf(expf(dt * A[j]), S[j], dx * B[j]);  // (lanes beyond the states: A, B and S are zero)
+      S[j] = fmaf(exp2_fast(dt * A[j]), S[j], dx * B[j]);  // (lanes beyond the states: A, B and S are zero)
       acc = fmaf(S[j], C[j], acc);
     }
     if (PASS != 1) {
@@ -263,8 +332,8 @@ struct GlaArgs {
   const void* v;
   int qkv_dtype;
   int q_stride, k_stride, v_stride;
-  const float* zd;  // [tokens, heads * key_dim]: the decays before the sigmoid
-  float inv_tau, scale;
+  const float* zd;  // [tokens, heads * key_dim]: the logarithms of the decays (nnis_gla_decays)
+  float scale;
   float* state;  // [slots, heads, key_dim, value_dim]
   const int* seq_slot;
   const int* seq_start;
@@ -281,7 +350,7 @@ struct GlaArgs {
 // decays' logarithms; 3 a piece from the state that the carry kernel left for it, writing the outputs.
 template <int GROUPS, int PASS>
 __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr int kCols = 4 * (kWave / GROUPS);  // value columns of a block (4 waves)
   const int b = blockIdx.z / a.pieces, piece = blockIdx.z % a.pieces, head = blockIdx.y;
   const int slot = a.seq_slot[b];
@@ -322,14 +391,14 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
       const int t = t0 + i / d, ch = i % d;
       if (PASS != 1) qs[i] = load_as_f32(a.q, a.qkv_dtype, (size_t)t * a.q_stride + head * d + ch) * a.scale;
       ks[i] = load_as_f32(a.k, a.qkv_dtype, (size_t)t * a.k_stride + head * d + ch);
-      as[i] = expf(log_sigmoid_f(a.zd[((size_t)t * a.heads + head) * d + ch]) * a.inv_tau);
+      as[i] = exp2_fast(a.zd[((size_t)t * a.heads + head) * d + ch] * kLog2e);
     }
     for (int i = threadIdx.x; i < count * kCols; i += blockDim.x) {
       const int t = t0 + i / kCols, cl = blockIdx.x * kCols + i % kCols;
       vs[i] = cl < e ? load_as_f32(a.v, a.qkv_dtype, (size_t)t * a.v_stride + head * e + cl) : 0.0f;
     }
     if (PASS == 1 && blockIdx.x == 0 && (int)threadIdx.x < d) {
-      for (int j = 0; j < count; ++j) log_sum += log_sigmoid_f(a.zd[((size_t)(t0 + j) * a.heads + head) * d + threadIdx.x]) * a.inv_tau;
+      for (int j = 0; j < count; ++j) log_sum += a.zd[((size_t)(t0 + j) * a.heads + head) * d + threadIdx.x];
     }
     __syncthreads();
     for (int j = 0; j < count; ++j) {
@@ -338,11 +407,27 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
       const float* kj = ks + j * d + group * 16;
       const float* aj = as + j * d + group * 16;
       float acc = 0.0f;
+      if (group * 16 + 16 <= d && d % 4 == 0) {  // whole rows of this group: 16 bytes a read
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if (group * 16 + r < d) {
-          S[r] = fmaf(aj[r], S[r], kj[r] * v);
-          if (PASS != 1) acc = fmaf(S[r], qj[r], acc);
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const float4 a4 = *(const float4*)(aj + 4 * r4), k4 = *(const float4*)(kj + 4 * r4);
+          const float av[4] = {a4.x, a4.y, a4.z, a4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) S[4 * r4 + i] = fmaf(av[i], S[4 * r4 + i], kv[i] * v);
+          if (PASS != 1) {
+            const float4 q4 = *(const float4*)(qj + 4 * r4);
+            const float qv[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = fmaf(S[4 * r4 + i], qv[i], acc);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (group * 16 + r < d) {
+            S[r] = fmaf(aj[r], S[r], kj[r] * v);
+            if (PASS != 1) acc = fmaf(S[r], qj[r], acc);
+          }
         }
       }
       if (PASS != 1) {
@@ -412,7 +497,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 
 extern "C" int nnis_conv_silu(const void* x, int x_dtype, int x_stride, const void* weight, const void* bias, int weight_dtype,
                               float* state, const int* tok_slot, const int* tok_pos, const int* seq_slot, const int* seq_start,
-                              int tokens, int batch, int channels, int taps, void* y, int y_dtype, void* stream) {
+                              int tokens, int batch, int channels, int taps, void* y, int y_dtype, int single, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(y_dtype), "conv: unknown dtype");
   NNIS_REQUIRE(taps >= 1 && taps <= kMostTaps, "conv: 1 to %d taps are taken, got %d", kMostTaps, taps);
   NNIS_REQUIRE(channels > 0 && x_stride >= channels && tokens >= 0 && batch >= 0, "conv: bad sizes");
@@ -422,10 +507,16 @@ extern "C" int nnis_conv_silu(const void* x, int x_dtype, int x_stride, const vo
   a.x = x; a.x_dtype = x_dtype; a.x_stride = x_stride; a.weight = weight; a.bias = bias; a.weight_dtype = weight_dtype; a.state = state;
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.seq_slot = seq_slot; a.seq_start = seq_start; a.tokens = tokens; a.batch = batch;
   a.channels = channels; a.taps = taps; a.y = y; a.y_dtype = y_dtype;
-  const size_t total = (size_t)tokens * channels;
-  size_t blocks = (total + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+  NNIS_REQUIRE(batch <= 65535 && (tokens + kConvStrip - 1) / kConvStrip <= 65535, "conv: too many rows or sequences for the grid");
+  const int width = channels >= 256 ? 256 : 64;
+  if (single) {  // every sequence brings one token: row b is sequence b's
+    NNIS_REQUIRE(tokens == batch, "conv: a step of single tokens has as many rows as sequences (%d and %d)", tokens, batch);
+    hipLaunchKernelGGL(conv_single_kernel, dim3((channels + width - 1) / width, batch), dim3(width), 0, (hipStream_t)stream, a);
+    NNIS_LAUNCH_CHECK("conv_single");
+    return 0;
+  }
+  hipLaunchKernelGGL(conv_silu_kernel, dim3((channels + width - 1) / width, (tokens + kConvStrip - 1) / kConvStrip), dim3(width), 0,
+                     (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("conv_silu");
   if (taps > 1) {
     const int threads = channels >= 256 ? 256 : 64;
@@ -481,13 +572,12 @@ extern "C" int nnis_selective_scan(const void* x, int x_dtype, const float* dt_p
 // piece, pieces: as nnis_selective_scan's (`carried`: batch * pieces * heads * key_dim * value_dim floats, `decayed`:
 // batch * pieces * heads * key_dim)
 extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qkv_dtype, int q_stride, int k_stride, int v_stride,
-                             const float* zd, float tau, float scale, float* state, const int* seq_slot, const int* seq_start,
+                             const float* zd, float scale, float* state, const int* seq_slot, const int* seq_start,
                              int batch, int heads, int key_dim, int value_dim, float* out, int piece, int pieces, float* carried,
                              float* decayed, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype), "gla_scan: unknown dtype %d", qkv_dtype);
   NNIS_REQUIRE(heads > 0 && key_dim > 0 && key_dim <= 256 && value_dim > 0 && batch >= 0,
                "gla_scan: bad sizes (heads %d, key channels %d: up to 256 are taken, value channels %d)", heads, key_dim, value_dim);
-  NNIS_REQUIRE(tau > 0.0f, "gla_scan: tau must be positive, got %g", (double)tau);
   NNIS_REQUIRE(q && k && v && zd && state && seq_slot && seq_start && out, "gla_scan: a pointer is missing");
   NNIS_REQUIRE(pieces <= 1 || (piece > 0 && carried && decayed), "gla_scan: pieces need their length and scratch");
   if (pieces < 1) pieces = 1;
@@ -495,7 +585,7 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
   if (batch == 0) return 0;
   GlaArgs a;
   a.q = q; a.k = k; a.v = v; a.qkv_dtype = qkv_dtype; a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.zd = zd;
-  a.inv_tau = 1.0f / tau; a.scale = scale; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads;
+  a.scale = scale; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.heads = heads;
   a.key_dim = key_dim; a.value_dim = value_dim; a.out = out; a.piece = piece; a.pieces = pieces; a.carried = carried; a.decayed = decayed;
   const int need = (key_dim + 15) / 16;
   const int groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
@@ -526,6 +616,24 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
   }
 #undef NNIS_GLA
   NNIS_LAUNCH_CHECK("gla_scan");
+  return 0;
+}
+
+// z[t, i] <- log(sigmoid(z[t, i] + bias[i])) / tau, in place: the logarithm of the decay sigmoid(.)^(1 / tau)
+__global__ void gla_decays_kernel(float* __restrict__ z, const float* __restrict__ bias, int width, size_t total, float inv_tau) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    z[i] = log_sigmoid_f(z[i] + bias[i % width]) * inv_tau;
+}
+
+extern "C" int nnis_gla_decays(float* z, const float* bias, int tokens, int width, float tau, void* stream) {
+  NNIS_REQUIRE(z && bias && tokens >= 0 && width > 0, "gla_decays: bad arguments");
+  NNIS_REQUIRE(tau > 0.0f, "gla_decays: tau must be positive, got %g", (double)tau);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * width;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(gla_decays_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, z, bias, width, total, 1.0f / tau);
+  NNIS_LAUNCH_CHECK("gla_decays");
   return 0;
 }
 

@@ -271,12 +271,38 @@ __global__ void gated_act_kernel(const void* __restrict__ gate_up, int in_dtype,
   }
 }
 
+// the same on bfloat16 rows whose width is a multiple of 8: 16-byte accesses, 8 channels a thread
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_r;
+
+__global__ void gated_act_bf16_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int inner, size_t groups, int act) {
+  const int per_row = inner / 8;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t row = i / per_row;
+    const int col = (int)(i % per_row) * 8;
+    const bf16x8_r g = *(const bf16x8_r*)(gate_up + row * 2 * inner + col);
+    const bf16x8_r u = *(const bf16x8_r*)(gate_up + row * 2 * inner + inner + col);
+    bf16x8_r y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (__bf16)(gate_activation((float)g[e], act) * (float)u[e]);
+    *(bf16x8_r*)(out + row * inner + col) = y;
+  }
+}
+
 extern "C" int nnis_gated_act(const void* gate_up, int in_dtype, void* out, int out_dtype, int tokens, int inner, int act,
                               void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(in_dtype) && nnis_dtype_ok(out_dtype), "gated_act: unknown dtype");
   NNIS_REQUIRE(tokens >= 0 && inner > 0, "gated_act: bad sizes tokens=%d inner=%d", tokens, inner);
   NNIS_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation %d", act);
   if (tokens == 0) return 0;
+  if (in_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && inner % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t groups = (size_t)tokens * (inner / 8);
+    size_t wide_blocks = (groups + 255) / 256;
+    if (wide_blocks > 65536) wide_blocks = 65536;
+    hipLaunchKernelGGL(gated_act_bf16_kernel, dim3((unsigned)wide_blocks), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)gate_up,
+                       (bf16_t*)out, inner, groups, act);
+    NNIS_LAUNCH_CHECK("gated_act_bf16");
+    return 0;
+  }
   const size_t total = (size_t)tokens * inner;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;

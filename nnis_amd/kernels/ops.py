@@ -73,11 +73,12 @@ _ATTN_SIGNATURES = {
 
 _RECURRENT_SIGNATURES = {
     "nnis_conv_silu": [_VOID, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT,
-                       _VOID],
+                       _INT, _VOID],
     "nnis_selective_scan": [_VOID, _INT, _VOID, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT,
                             _VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID],
-    "nnis_gla_scan": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _FLT, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT,
+    "nnis_gla_scan": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _FLT, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT,
                       _VOID, _INT, _INT, _VOID, _VOID, _VOID],
+    "nnis_gla_decays": [_VOID, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
 }
 
@@ -1303,7 +1304,8 @@ def conv_silu(x: torch.Tensor, channels: int, weight: torch.Tensor, bias: Option
     lib = recurrent()
     _check(lib, lib.nnis_conv_silu(x.data_ptr(), _code(x), x.stride(0), weight.data_ptr(), _ptr(bias), _code(weight), _ptr(state),
                                    ctx.tok_slot.data_ptr(), ctx.tok_pos.data_ptr(), ctx.seq_slot.data_ptr(), ctx.seq_start.data_ptr(),
-                                   tokens, ctx.batch, channels, taps, out.data_ptr(), _code(out), _stream()))
+                                   tokens, ctx.batch, channels, taps, out.data_ptr(), _code(out),
+                                   1 if (ctx.decode and tokens == ctx.batch) else 0, _stream()))
     return out
 
 
@@ -1339,12 +1341,24 @@ def selective_scan(x: torch.Tensor, dt_pre: torch.Tensor, bc: torch.Tensor, z: t
     return out
 
 
-def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logits: torch.Tensor, tau: float, scale: float,
+def gla_decays(logits: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Tensor:
+    """In place: logits <- log(sigmoid(logits + bias)) / tau, the logarithms of the decays sigmoid(.)^(1 / tau) that
+    ``gla_scan`` takes.  Both float32; ``bias`` has one entry per column."""
+    _dev(logits, "logits"), _dev(bias, "bias")
+    if logits.dtype != torch.float32 or bias.dtype != torch.float32 or logits.dim() != 2 or bias.numel() != logits.shape[1]:
+        raise KernelError("gla_decays: logits must be float32 [tokens, channels] and the bias float32 [channels]")
+    lib = recurrent()
+    _check(lib, lib.nnis_gla_decays(logits.data_ptr(), bias.data_ptr(), logits.shape[0], logits.shape[1], float(tau), _stream()))
+    return logits
+
+
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logs: torch.Tensor, scale: float,
              state: torch.Tensor, ctx, heads: int, out: torch.Tensor) -> torch.Tensor:
     """Gated linear attention over each sequence's tokens, from and into ``state`` (float32 [slots, heads, key
-    channels, value channels]): alpha = sigmoid(decay_logits)^(1 / tau); S <- diag(alpha) S + k v^T; out = S^T
-    (q * scale), raw, float32 [tokens, heads * value channels].  q, k [tokens, heads * key channels] and v are views
-    whose rows may be further apart; ``decay_logits`` float32 [tokens, heads * key channels]."""
+    channels, value channels]): alpha = exp(decay_logs); S <- diag(alpha) S + k v^T; out = S^T (q * scale), raw,
+    float32 [tokens, heads * value channels].  q, k [tokens, heads * key channels] and v are views whose rows may be
+    further apart; ``decay_logs`` float32 [tokens, heads * key channels] (``gla_decays``)."""
+    decay_logits = decay_logs
     tokens = q.shape[0]
     key_dim, value_dim = q.shape[1] // heads, v.shape[1] // heads
     for t, what in ((q, "q"), (k, "k"), (v, "v")):
@@ -1368,7 +1382,7 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay_logits: to
         decayed = torch.empty(ctx.batch * pieces * heads * key_dim, dtype=torch.float32, device=out.device)
     lib = recurrent()
     _check(lib, lib.nnis_gla_scan(q.data_ptr(), k.data_ptr(), v.data_ptr(), _code(q), stride(q), stride(k), stride(v),
-                                  decay_logits.data_ptr(), float(tau), float(scale), state.data_ptr(), ctx.seq_slot.data_ptr(),
+                                  decay_logits.data_ptr(), float(scale), state.data_ptr(), ctx.seq_slot.data_ptr(),
                                   ctx.seq_start.data_ptr(), ctx.batch, heads, key_dim, value_dim, out.data_ptr(), piece, pieces,
                                   _ptr(carried), _ptr(decayed), _stream()))
     return out

@@ -158,10 +158,10 @@ class GatedLinearAttention(Mixer):
         tokens = x.shape[0]
         qkvg = self.qkvg(x, rt)
         logits = self.a2(self.a1(x, rt), rt, out_dtype=torch.float32)
-        rt.ops.add_bias(logits, self.a2_bias)
+        rt.ops.gla_decays(logits, self.a2_bias, self.tau)  # the decays' logarithms, once for all heads' blocks
         q, k = qkvg[:, :H * d], qkvg[:, H * d:2 * H * d]
         v, g = qkvg[:, 2 * H * d:2 * H * d + H * e], qkvg[:, 2 * H * d + H * e:]
-        o = rt.ops.gla_scan(q, k, v, logits, self.tau, d ** -0.5, view.state, ctx, H, rt.empty(tokens, H * e, dtype=torch.float32))
+        o = rt.ops.gla_scan(q, k, v, logits, d ** -0.5, view.state, ctx, H, rt.empty(tokens, H * e, dtype=torch.float32))
         gated = rt.ops.head_norm_gate(o, g, self.norm, self.eps, H, rt.empty(tokens, H * e))
         return self.out(gated, rt)
 

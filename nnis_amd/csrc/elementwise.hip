@@ -384,9 +384,21 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
   if (slot < 0) return;
   const int pos = a.tok_pos[token];
   const int hd = a.head_dim;
+  const int vd = a.value_dim;
   const int half = a.rot_dim / 2;
-  const int row_width = (a.heads + 2 * a.kv_heads) * hd;
+  const int row_width = (a.heads + a.kv_heads) * hd + a.kv_heads * vd;
   const bf16_t* src = (const bf16_t*)a.qkv + (size_t)token * row_width;
+  const bf16_t* bias = (const bf16_t*)a.bias;  // bfloat16 here, or null
+  // 4 channels from column `at` of the token's row, with their bias, in 32-bit
+  auto four = [&](size_t at) {
+    const bf16x4_t x = *(const bf16x4_t*)(src + at);
+    f32x4_t f = {(float)x[0], (float)x[1], (float)x[2], (float)x[3]};
+    if (bias) {
+      const bf16x4_t b = *(const bf16x4_t*)(bias + at);
+      f += (f32x4_t){(float)b[0], (float)b[1], (float)b[2], (float)b[3]};
+    }
+    return f;
+  };
   const bool rotate = a.cos_table != nullptr && pos < a.table_positions;
   int page = -1;
   if (a.k_pages) page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
@@ -394,7 +406,7 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
   const int rot_heads = a.heads + a.kv_heads;
   const int groups_per_head = (hd - half) / 4;  // half/4 groups of pairs, then (hd - rot_dim)/4 pass-through groups
   const int rot_items = rot_heads * groups_per_head;
-  const int v_items = page >= 0 ? a.kv_heads * (hd / 4) : 0;
+  const int v_items = page >= 0 ? a.kv_heads * (vd / 4) : 0;
   for (int item = threadIdx.x; item < rot_items + v_items; item += blockDim.x) {
     if (item < rot_items) {
       const int head = item / groups_per_head;
@@ -409,9 +421,9 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
         k_page = (bf16_t*)a.k_pages + ((size_t)page * a.kv_heads + (head - a.heads)) * nnis_k_page_elems(hd);
       }
       auto place = [&](int ch) { return q_row ? q_row + ch : k_page + nnis_k_offset(in_page, ch); };
-      const bf16_t* x = src + (size_t)head * hd;
+      const size_t x = (size_t)head * hd;
       if (e < half) {
-        const bf16x4_t x0 = *(const bf16x4_t*)(x + e), x1 = *(const bf16x4_t*)(x + e + half);
+        const f32x4_t x0 = four(x + e), x1 = four(x + e + half);
         f32x4_t c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
         if (rotate) {
           c = *(const f32x4_t*)(a.cos_table + (size_t)pos * half + e);
@@ -420,23 +432,27 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
         bf16x4_t lo, hi;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float f0 = (float)x0[j], f1 = (float)x1[j];
+          const float f0 = x0[j], f1 = x1[j];
           lo[j] = (__bf16)(f0 * c[j] - f1 * sn[j]);
           hi[j] = (__bf16)(f1 * c[j] + f0 * sn[j]);
         }
         *(bf16x4_t*)place(e) = lo;
         *(bf16x4_t*)place(e + half) = hi;
       } else {
-        *(bf16x4_t*)place(e + half) = *(const bf16x4_t*)(x + e + half);  // channels at and beyond rot_dim
+        const f32x4_t f = four(x + e + half);  // channels at and beyond rot_dim
+        bf16x4_t through;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) through[j] = (__bf16)f[j];
+        *(bf16x4_t*)place(e + half) = through;
       }
     } else {
       const int v_item = item - rot_items;
-      const int kv_head = v_item / (hd / 4);
-      const int d = (v_item % (hd / 4)) * 4;
-      const bf16x4_t v = *(const bf16x4_t*)(src + (size_t)(a.heads + a.kv_heads + kv_head) * hd + d);
-      bf16_t* dst = (bf16_t*)a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(hd);
+      const int kv_head = v_item / (vd / 4);
+      const int d = (v_item % (vd / 4)) * 4;
+      const f32x4_t v = four((size_t)(a.heads + a.kv_heads) * hd + (size_t)kv_head * vd + d);
+      bf16_t* dst = (bf16_t*)a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(vd);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dst[nnis_v_offset(d + j, in_page)] = v[j];
+      for (int j = 0; j < 4; ++j) dst[nnis_v_offset(d + j, in_page)] = (__bf16)v[j];
     }
   }
 }
@@ -469,8 +485,9 @@ extern "C" int nnis_rope_kv_write_wide(const void* qkv, int qkv_dtype, void* q_o
   const bool all_bf16 = qkv_dtype == NNIS_BF16 && q_dtype == NNIS_BF16 && (k_pages == nullptr || cache_dtype == NNIS_BF16);
   const bool aligned = ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)q_out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
                        ((uintptr_t)v_pages % 16 == 0) && ((uintptr_t)cos_table % 16 == 0) && ((uintptr_t)sin_table % 16 == 0);
-  if (all_bf16 && aligned && head_dim % 4 == 0 && (a.rot_dim / 2) % 4 == 0 && value_dim == head_dim && bias == nullptr) {
-    const int items = (heads + kv_heads) * (head_dim - a.rot_dim / 2) / 4 + kv_heads * head_dim / 4;
+  if (all_bf16 && aligned && head_dim % 4 == 0 && (a.rot_dim / 2) % 4 == 0 && value_dim % 4 == 0 &&
+      (bias == nullptr || (bias_dtype == NNIS_BF16 && (uintptr_t)bias % 8 == 0))) {
+    const int items = (heads + kv_heads) * (head_dim - a.rot_dim / 2) / 4 + kv_heads * value_dim / 4;
     const int threads = items > 128 ? 256 : (items > 64 ? 128 : 64);
     hipLaunchKernelGGL(rope_kv_write_bf16_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
     NNIS_LAUNCH_CHECK("rope_kv_write_bf16");

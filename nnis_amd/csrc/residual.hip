@@ -157,6 +157,111 @@ __global__ void stream_kernel(StreamArgs a) {
   }
 }
 
+// The same with a row in registers: a thread takes CH pieces of 4 channels of every stream, asks for all of them at
+// once (the loop above waits for memory once a piece), and keeps u in registers.  Widths in steps of 4 up to
+// 4096 * CH... channels a block of up to 1024 threads covers.
+typedef __attribute__((ext_vector_type(4))) float f32x4_r;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_r;
+
+__device__ __forceinline__ f32x4_r load4_r(const void* base, int dtype, size_t index) {
+  if (dtype == NNIS_F32) return *(const f32x4_r*)((const float*)base + index);
+  const bf16x4_r v = *(const bf16x4_r*)((const bf16_t*)base + index);
+  return (f32x4_r){(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+__device__ __forceinline__ void store4_r(void* base, int dtype, size_t index, f32x4_r v) {
+  if (dtype == NNIS_F32) {
+    *(f32x4_r*)((float*)base + index) = v;
+  } else {
+    bf16x4_r packed;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)v[e];
+    *(bf16x4_r*)((bf16_t*)base + index) = packed;
+  }
+}
+
+template <int CH, int SMAX>
+__global__ __launch_bounds__(1024) void stream_wide_kernel(StreamArgs a) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int row = a.rows ? a.rows[out_row] : out_row;
+  const int S = a.streams;
+  const size_t plane = (size_t)a.tokens * a.width;
+  float* x = a.x + (size_t)row * a.width;
+  f32x4_r v[SMAX][CH], y[CH];
+  bool inside[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int col = 4 * (threadIdx.x + i * blockDim.x);
+    inside[i] = col < a.width;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) v[s][i] = (inside[i] && s < S) ? *(const f32x4_r*)(x + s * plane + col) : (f32x4_r){0.0f, 0.0f, 0.0f, 0.0f};
+    y[i] = (a.y && inside[i]) ? load4_r(a.y, a.y_dtype, (size_t)row * a.width + col) : (f32x4_r){0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  float take[SMAX];
+#pragma unroll
+  for (int s = 0; s < SMAX; ++s) take[s] = s < S ? (a.take ? a.take[s] : 1.0f) : 0.0f;
+  if (a.y) {
+    float mix[SMAX][SMAX], gain[SMAX];
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+      gain[s] = s < S ? a.gain[s] : 0.0f;
+#pragma unroll
+      for (int t = 0; t < SMAX; ++t) mix[s][t] = (s < S && t < S) ? a.mix[s * S + t] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      f32x4_r w[SMAX];
+#pragma unroll
+      for (int t = 0; t < SMAX; ++t) {
+        w[t] = gain[t] * y[i];
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) w[t] += mix[s][t] * v[s][i];
+      }
+#pragma unroll
+      for (int t = 0; t < SMAX; ++t) {
+        v[t][i] = w[t];
+        if (inside[i] && t < S) *(f32x4_r*)(x + t * plane + 4 * (threadIdx.x + i * blockDim.x)) = w[t];
+      }
+    }
+  }
+  if (a.h == nullptr) return;
+  f32x4_r u[CH];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    u[i] = (f32x4_r){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) u[i] += take[s] * v[s][i];
+    sum += (u[i][0] + u[i][1]) + (u[i][2] + u[i][3]);
+  }
+  const size_t out_base = (size_t)out_row * a.width;
+  float mean = 0.0f, scale = 1.0f;
+  if (a.weight) {
+    const float inv_width = 1.0f / (float)a.width;
+    if (a.centred) mean = block_sum(sum, scratch) * inv_width;
+    float squares = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+      if (inside[i]) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) squares = fmaf(u[i][e] - mean, u[i][e] - mean, squares);
+      }
+    scale = 1.0f / sqrtf(block_sum(squares, scratch) * inv_width + a.eps);
+  }
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int col = 4 * (threadIdx.x + i * blockDim.x);
+    if (!inside[i]) continue;
+    f32x4_r out = u[i];
+    if (a.weight) {
+      out = ((u[i] - mean) * scale) * load4_r(a.weight, a.weight_dtype, col);
+      if (a.bias) out += load4_r(a.bias, a.weight_dtype, col);
+    }
+    store4_r(a.h, a.h_dtype, out_base + col, out);
+  }
+}
+
 extern "C" int nnis_stream_step(float* x, int streams, int tokens, int width, const void* y, int y_dtype, const float* mix,
                                 const float* gain, const float* take, const void* weight, const void* bias, int weight_dtype,
                                 int centred, float eps, void* h, int h_dtype, const int* rows, int out_rows, void* stream) {
@@ -174,6 +279,23 @@ extern "C" int nnis_stream_step(float* x, int streams, int tokens, int width, co
   a.x = x; a.streams = streams; a.tokens = tokens; a.width = width; a.y = y; a.y_dtype = y_dtype; a.mix = mix; a.gain = gain;
   a.take = take; a.weight = weight; a.bias = bias; a.weight_dtype = weight_dtype; a.centred = centred; a.eps = eps; a.h = h;
   a.h_dtype = h_dtype; a.rows = rows;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)h % 16 == 0) && ((uintptr_t)weight % 16 == 0) &&
+                       ((uintptr_t)bias % 16 == 0);
+  if (width % 4 == 0 && aligned && width / 4 <= 2048) {
+    const int pieces = width / 4;
+    const int per = pieces > 1024 ? 2 : 1;
+    const int block = ((pieces + per - 1) / per + 63) / 64 * 64;
+    hipStream_t s = (hipStream_t)stream;
+    if (streams <= 4) {
+      if (per == 1) hipLaunchKernelGGL((stream_wide_kernel<1, 4>), dim3(out_rows), dim3(block), 0, s, a);
+      else hipLaunchKernelGGL((stream_wide_kernel<2, 4>), dim3(out_rows), dim3(block), 0, s, a);
+    } else {
+      if (per == 1) hipLaunchKernelGGL((stream_wide_kernel<1, kMostStreams>), dim3(out_rows), dim3(block), 0, s, a);
+      else hipLaunchKernelGGL((stream_wide_kernel<2, kMostStreams>), dim3(out_rows), dim3(block), 0, s, a);
+    }
+    NNIS_LAUNCH_CHECK("stream_step");
+    return 0;
+  }
   const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
   hipLaunchKernelGGL(stream_kernel, dim3(out_rows), dim3(threads), (size_t)width * sizeof(float), (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("stream_step");
@@ -230,6 +352,33 @@ __global__ void branch_mean_kernel(BranchArgs a) {
   }
 }
 
+// with a row in registers (as stream_wide_kernel): widths in steps of 4 up to 4096 channels
+__global__ __launch_bounds__(1024) void branch_mean_wide_kernel(BranchArgs a) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * a.width;
+  const int col = 4 * threadIdx.x;
+  const bool inside = col < a.width;
+  f32x4_r v[kMostBranches];
+  float squares[kMostBranches];
+#pragma unroll
+  for (int i = 0; i < kMostBranches; ++i) {
+    v[i] = (f32x4_r){0.0f, 0.0f, 0.0f, 0.0f};
+    if (i < a.count && inside) {
+      v[i] = load4_r(a.y[i], a.y_dtype, base + col);
+      if (a.bias[i]) v[i] += load4_r(a.bias[i], a.weight_dtype, col);
+    }
+    squares[i] = (v[i][0] * v[i][0] + v[i][1] * v[i][1]) + (v[i][2] * v[i][2] + v[i][3] * v[i][3]);
+  }
+  f32x4_r acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int i = 0; i < kMostBranches; ++i)
+    if (i < a.count) {
+      const float scale = 1.0f / sqrtf(block_sum(squares[i], scratch) / (float)a.width + a.eps);
+      if (inside) acc += (v[i] * scale) * load4_r(a.weight[i], a.weight_dtype, col);
+    }
+  if (inside) store4_r(a.out, a.out_dtype, base + col, acc * (1.0f / (float)a.count));
+}
+
 extern "C" int nnis_branch_mean(const void* const* y, const void* const* weight, const void* const* bias, int count, int y_dtype,
                                 int weight_dtype, int tokens, int width, float eps, void* out, int out_dtype, void* stream) {
   NNIS_REQUIRE(count >= 1 && count <= kMostBranches, "branch_mean: 1 to %d branches are taken, got %d", kMostBranches, count);
@@ -244,6 +393,14 @@ extern "C" int nnis_branch_mean(const void* const* y, const void* const* weight,
     NNIS_REQUIRE(i >= count || (a.y[i] && a.weight[i]), "branch_mean: branch %d has no input or no weight", i);
   }
   a.count = count; a.y_dtype = y_dtype; a.weight_dtype = weight_dtype; a.width = width; a.eps = eps; a.out = out; a.out_dtype = out_dtype;
+  bool aligned = (uintptr_t)out % 16 == 0;
+  for (int i = 0; i < count; ++i)
+    aligned = aligned && (uintptr_t)a.y[i] % 16 == 0 && (uintptr_t)a.weight[i] % 16 == 0 && (uintptr_t)a.bias[i] % 16 == 0;
+  if (width % 4 == 0 && aligned && width / 4 <= 1024) {
+    hipLaunchKernelGGL(branch_mean_wide_kernel, dim3(tokens), dim3((width / 4 + 63) / 64 * 64), 0, (hipStream_t)stream, a);
+    NNIS_LAUNCH_CHECK("branch_mean");
+    return 0;
+  }
   const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
   hipLaunchKernelGGL(branch_mean_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
   NNIS_LAUNCH_CHECK("branch_mean");

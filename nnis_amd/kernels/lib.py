@@ -50,7 +50,7 @@ FLAGS = [
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 PREBUILT_HEAD_DIMS = (6, 16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 # values of another size than the keys: what the tests use
-PREBUILT_WIDE_VALUES = ("attn_hd32v16c", "attn_hd16v48c", "attn_hd48v64c", "attn_hd64v32c", "attn_hd6v10c", "attn_hd32c", "attn_hd64c",
+PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_hd48v64c", "attn_hd64v32c", "attn_hd6v10c", "attn_hd32c", "attn_hd64c",
                         "attn_hd16c", "attn_hd128c", "attn_hd128v64c")
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -153,8 +153,8 @@ ATTENTION_MOST_CHANNELS = 256
 
 def attention_check(head_dim: int, value_dim: Optional[int] = None) -> None:
     """Raises ``Unsupported`` for a head size that no attention kernel here takes."""
-    if head_dim <= 0 or head_dim % 2 != 0 or head_dim > ATTENTION_MOST_CHANNELS:
-        raise Unsupported(f"the attention kernels take an even head_dim up to {ATTENTION_MOST_CHANNELS}, got {head_dim}")
+    if head_dim <= 0 or head_dim > ATTENTION_MOST_CHANNELS:
+        raise Unsupported(f"the attention kernels take a head_dim up to {ATTENTION_MOST_CHANNELS}, got {head_dim}")
     if value_dim is not None and value_dim != head_dim and not 0 < value_dim <= ATTENTION_MOST_CHANNELS:
         raise Unsupported(f"the attention kernels take values of up to {ATTENTION_MOST_CHANNELS} channels, got {value_dim}")
 

@@ -21,7 +21,7 @@ from zifunex_configs import ZIFUNEX_CONFIGS, attention, gla, parallel, scan, zif
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
-HEAD_SIZES = [(32, 16), (16, 48), (48, 64), (64, 32), (32, 32), (64, 64), (16, 16), (6, 10)]  # (key, value) channels of a head
+HEAD_SIZES = [(7, 5), (32, 16), (16, 48), (48, 64), (64, 32), (32, 32), (64, 64), (16, 16), (6, 10)]  # (key, value) channels of a head
 
 
 def _relative(got, want):

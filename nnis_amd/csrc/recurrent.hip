@@ -19,7 +19,14 @@ constexpr float kLog2e = 1.4426950408889634f;
 // two of a product that is made once, exp(dt A) = 2^(dt (A log2 e))
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.0f + exp2_fast(-z * kLog2e)); }
-__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+// log(1 + e^z) by the hardware's 2^x and log2: e^z itself where it is small (the sum 1 + e^z would round it away;
+// three terms of the logarithm's series keep a relative error of e^3z / 4 < 2e-6 below e^z = 0.02), z where it is large
+__device__ __forceinline__ float softplus_f(float z) {
+  const float t = exp2_fast(z * kLog2e);
+  const float small = t * (1.0f - t * (0.5f - t * (1.0f / 3.0f)));
+  const float mid = __builtin_amdgcn_logf(1.0f + t) * 0.6931471805599453f;
+  return z > 20.0f ? z : (t < 0.02f ? small : mid);
+}
 // log(sigmoid(z)) = min(z, 0) - log(1 + exp(-|z|))
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
@@ -72,8 +79,14 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
     held[j] = 0.0f;
   }
   const float bias = a.bias ? load_as_f32(a.bias, a.weight_dtype, c) : 0.0f;
+  float fresh[kConvStrip];  // the strip's own inputs, all asked for at once
+#pragma unroll
+  for (int i = 0; i < kConvStrip; ++i) fresh[i] = begin + i < end ? load_as_f32(a.x, a.x_dtype, (size_t)(begin + i) * a.x_stride + c) : 0.0f;
   int before = -2;  // the slot of the row before, if its inputs are held
-  for (int token = begin; token < end; ++token) {
+#pragma unroll
+  for (int i = 0; i < kConvStrip; ++i) {
+    const int token = begin + i;
+    if (token >= end) break;
     const int slot = a.tok_slot[token];
     if (slot < 0) {
       store_from_f32(a.y, a.y_dtype, (size_t)token * a.channels + c, 0.0f);
@@ -84,10 +97,9 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(ConvArgs a) {
 #pragma unroll
       for (int j = 0; j + 1 < kMostTaps; ++j)
         if (j + 1 < a.taps) held[j] = held[j + 1];
-      const float now = load_as_f32(a.x, a.x_dtype, (size_t)token * a.x_stride + c);
 #pragma unroll
       for (int j = 0; j < kMostTaps; ++j)
-        if (j == a.taps - 1) held[j] = now;
+        if (j == a.taps - 1) held[j] = fresh[i];
     } else {
       const int pos = a.tok_pos[token];
       bool in_step = true;
@@ -201,6 +213,18 @@ struct ScanArgs {
 // (2) one thread a (channel, state) walks the pieces, I_0 = the sequence's state, I_(k+1) = exp(A sum_k) I_k + E_k,
 // and leaves I_k in E_k's place; (3) every piece runs again, from I_k, and writes the outputs; the last one leaves
 // the sequence's state.  PASS 0 is the plain run of a whole sequence by one block (single tokens, short runs).
+// a lane's 8 of a token's `n` values from `row`: two 16-byte loads where the row allows them
+__device__ __forceinline__ void load8(float (&into)[8], const float* row, int part, int n, bool wide) {
+  if (wide && part * 8 + 8 <= n) {  // (a lane beyond the states gets zeros below)
+    const float4 lo = *(const float4*)(row + part * 8), hi = *(const float4*)(row + part * 8 + 4);
+    into[0] = lo.x; into[1] = lo.y; into[2] = lo.z; into[3] = lo.w;
+    into[4] = hi.x; into[5] = hi.y; into[6] = hi.z; into[7] = hi.w;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) into[j] = part * 8 + j < n ? row[part * 8 + j] : 0.0f;
+  }
+}
+
 template <int LANES, int PASS>
 __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   const int b = blockIdx.z, piece = blockIdx.y;
@@ -237,12 +261,11 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   float dt_next = a.dt_pre[(size_t)first * a.channels + cc];
   float z_next = PASS == 1 ? 0.0f : load_as_f32(a.z, a.z_dtype, (size_t)first * a.z_stride + cc);
   float B_next[8], C_next[8];
+  const bool wide = N % 8 == 0 && ((uintptr_t)a.bc % 16 == 0);  // a lane's 8 values lie within the row, on 16-byte boundaries
+  load8(B_next, a.bc + (size_t)first * 2 * N, part, N, wide);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int n = part * 8 + j;
-    B_next[j] = n < N ? a.bc[(size_t)first * 2 * N + n] : 0.0f;
-    C_next[j] = (PASS != 1 && n < N) ? a.bc[(size_t)first * 2 * N + N + n] : 0.0f;
-  }
+  for (int j = 0; j < 8; ++j) C_next[j] = 0.0f;
+  if (PASS != 1) load8(C_next, a.bc + (size_t)first * 2 * N + N, part, N, wide);
   for (int t = first; t < last; ++t) {
     const float x = x_next, z = z_next;
     // (the step size is the same in all lanes of a channel: one of them takes the logarithm)
@@ -258,14 +281,8 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
     x_next = load_as_f32(a.x, a.x_dtype, (size_t)ahead * a.channels + cc);
     dt_next = a.dt_pre[(size_t)ahead * a.channels + cc];
     if (PASS != 1) z_next = load_as_f32(a.z, a.z_dtype, (size_t)ahead * a.z_stride + cc);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int n = part * 8 + j;
-      if (n < N) {
-        B_next[j] = a.bc[(size_t)ahead * 2 * N + n];
-        if (PASS != 1) C_next[j] = a.bc[(size_t)ahead * 2 * N + N + n];
-      }
-    }
+    load8(B_next, a.bc + (size_t)ahead * 2 * N, part, N, wide);
+    if (PASS != 1) load8(C_next, a.bc + (size_t)ahead * 2 * N + N, part, N, wide);
     const float dx = dt * x;
     steps += dt;
     float acc = 0.0f;

@@ -181,8 +181,8 @@ __global__ void conv_state_kernel(ConvArgs a) {
 //   dt = softplus(dt_pre[t, c] + dt_bias[c])
 //   S[c, n] <- exp(dt * A[c, n]) S[c, n] + dt * x[t, c] * B[t, n]
 //   y[t, c] = (sum_n S[c, n] C[t, n] + D[c] x[t, c]) * silu(z[t, c])
-// A thread keeps 8 states of one channel; the lanes of a channel (a power of two, up to 16) sit side by side
-// and add their parts of y by lane exchanges.  bc [tokens, 2 * states]: B then C.  A = -exp(A_log) comes
+// A thread keeps 16 states of one channel (8 where there are no more); the lanes of a channel (a power of two, up to 8)
+// sit side by side and add their parts of y by lane exchanges.  bc [tokens, 2 * states]: B then C.  A = -exp(A_log) comes
 // ready-made.  state [slots, channels, states].
 // -----------------------------------------------------------------------------
 struct ScanArgs {
@@ -213,19 +213,23 @@ struct ScanArgs {
 // (2) one thread a (channel, state) walks the pieces, I_0 = the sequence's state, I_(k+1) = exp(A sum_k) I_k + E_k,
 // and leaves I_k in E_k's place; (3) every piece runs again, from I_k, and writes the outputs; the last one leaves
 // the sequence's state.  PASS 0 is the plain run of a whole sequence by one block (single tokens, short runs).
-// a lane's 8 of a token's `n` values from `row`: two 16-byte loads where the row allows them
-__device__ __forceinline__ void load8(float (&into)[8], const float* row, int part, int n, bool wide) {
-  if (wide && part * 8 + 8 <= n) {  // (a lane beyond the states gets zeros below)
-    const float4 lo = *(const float4*)(row + part * 8), hi = *(const float4*)(row + part * 8 + 4);
-    into[0] = lo.x; into[1] = lo.y; into[2] = lo.z; into[3] = lo.w;
-    into[4] = hi.x; into[5] = hi.y; into[6] = hi.z; into[7] = hi.w;
+// a lane's PER of a token's `n` values from `row`: 16-byte loads where the row allows them
+template <int PER>
+__device__ __forceinline__ void load_lane(float (&into)[PER], const float* row, int part, int n, bool wide) {
+  if (wide && part * PER + PER <= n) {  // (a lane that reaches beyond the states takes them one by one, zeros beyond)
+#pragma unroll
+    for (int q = 0; q < PER / 4; ++q) {
+      const float4 v = *(const float4*)(row + part * PER + 4 * q);
+      into[4 * q] = v.x; into[4 * q + 1] = v.y; into[4 * q + 2] = v.z; into[4 * q + 3] = v.w;
+    }
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) into[j] = part * 8 + j < n ? row[part * 8 + j] : 0.0f;
+    for (int j = 0; j < PER; ++j) into[j] = part * PER + j < n ? row[part * PER + j] : 0.0f;
   }
 }
 
-template <int LANES, int PASS>
+// PER: states a lane keeps (8, or 16: one lane a channel up to 16 states, half the lanes and none of the exchanges)
+template <int LANES, int PASS, int PER>
 __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   const int b = blockIdx.z, piece = blockIdx.y;
   const int slot = a.seq_slot[b];
@@ -244,12 +248,12 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   const bool live = c < a.channels;
   const int cc = live ? c : 0;
   const int N = a.states;
-  float S[8], A[8];
+  float S[PER], A[PER];
   float* state = a.state + ((size_t)slot * a.channels + cc) * N;
   float* carried = PASS == 0 ? nullptr : a.carried + (((size_t)b * a.pieces + piece) * a.channels + cc) * N;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int n = part * 8 + j;
+  for (int j = 0; j < PER; ++j) {
+    const int n = part * PER + j;
     const bool here = live && n < N;
     S[j] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[n] : carried[n]);
     A[j] = here ? a.A[(size_t)cc * N + n] * kLog2e : 0.0f;  // (in powers of two)
@@ -260,20 +264,20 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   float x_next = load_as_f32(a.x, a.x_dtype, (size_t)first * a.channels + cc);
   float dt_next = a.dt_pre[(size_t)first * a.channels + cc];
   float z_next = PASS == 1 ? 0.0f : load_as_f32(a.z, a.z_dtype, (size_t)first * a.z_stride + cc);
-  float B_next[8], C_next[8];
-  const bool wide = N % 8 == 0 && ((uintptr_t)a.bc % 16 == 0);  // a lane's 8 values lie within the row, on 16-byte boundaries
-  load8(B_next, a.bc + (size_t)first * 2 * N, part, N, wide);
+  float B_next[PER], C_next[PER];
+  const bool wide = N % 4 == 0 && ((uintptr_t)a.bc % 16 == 0);  // a lane's 8 values lie within the row, on 16-byte boundaries
+  load_lane<PER>(B_next, a.bc + (size_t)first * 2 * N, part, N, wide);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) C_next[j] = 0.0f;
-  if (PASS != 1) load8(C_next, a.bc + (size_t)first * 2 * N + N, part, N, wide);
+  for (int j = 0; j < PER; ++j) C_next[j] = 0.0f;
+  if (PASS != 1) load_lane<PER>(C_next, a.bc + (size_t)first * 2 * N + N, part, N, wide);
   for (int t = first; t < last; ++t) {
     const float x = x_next, z = z_next;
     // (the step size is the same in all lanes of a channel: one of them takes the logarithm)
     float dt = part == 0 ? softplus_f(dt_next + dt_bias) : 0.0f;
     if (LANES > 1) dt = __shfl(dt, (threadIdx.x % kWave) & ~(LANES - 1), kWave);
-    float B[8], C[8];
+    float B[PER], C[PER];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < PER; ++j) {
       B[j] = B_next[j];
       C[j] = C_next[j];
     }
@@ -281,13 +285,13 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
     x_next = load_as_f32(a.x, a.x_dtype, (size_t)ahead * a.channels + cc);
     dt_next = a.dt_pre[(size_t)ahead * a.channels + cc];
     if (PASS != 1) z_next = load_as_f32(a.z, a.z_dtype, (size_t)ahead * a.z_stride + cc);
-    load8(B_next, a.bc + (size_t)ahead * 2 * N, part, N, wide);
-    if (PASS != 1) load8(C_next, a.bc + (size_t)ahead * 2 * N + N, part, N, wide);
+    load_lane<PER>(B_next, a.bc + (size_t)ahead * 2 * N, part, N, wide);
+    if (PASS != 1) load_lane<PER>(C_next, a.bc + (size_t)ahead * 2 * N + N, part, N, wide);
     const float dx = dt * x;
     steps += dt;
     float acc = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < PER; ++j) {
       S[j] = fmaf(exp2_fast(dt * A[j]), S[j], dx * B[j]);  // (lanes beyond the states: A, B and S are zero)
       acc = fmaf(S[j], C[j], acc);
     }
@@ -305,8 +309,8 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(ScanArgs a) {
   }
   float* into = PASS == 1 ? carried : state;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int n = part * 8 + j;
+  for (int j = 0; j < PER; ++j) {
+    const int n = part * PER + j;
     if (n < N) into[n] = S[j];
   }
 }
@@ -323,13 +327,22 @@ __global__ void selective_scan_carry_kernel(ScanArgs a) {
   const int c = i / a.states;
   const float A = a.A[i];
   float I = a.state[(size_t)slot * a.channels * a.states + i];
-  for (int k = 0; k < pieces_here; ++k) {
-    float* at = a.carried + ((size_t)b * a.pieces + k) * a.channels * a.states + i;
-    const bool more = k + 1 < pieces_here;
-    const float E = more ? *at : 0.0f;
-    const float steps = more ? a.stepped[((size_t)b * a.pieces + k) * a.channels + c] : 0.0f;
-    *at = I;
-    I = fmaf(expf(A * steps), I, E);
+  const size_t per = (size_t)a.channels * a.states;
+  for (int k0 = 0; k0 < pieces_here; k0 += 8) {  // eight pieces' ends and steps asked for at once
+    float E[8], steps[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool more = k0 + j + 1 < pieces_here;
+      E[j] = more ? a.carried[((size_t)b * a.pieces + k0 + j) * per + i] : 0.0f;
+      steps[j] = more ? a.stepped[((size_t)b * a.pieces + k0 + j) * a.channels + c] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (k0 + j < pieces_here) {
+        a.carried[((size_t)b * a.pieces + k0 + j) * per + i] = I;
+        I = fmaf(expf(A * steps[j]), I, E[j]);
+      }
+    }
   }
 }
 
@@ -478,13 +491,21 @@ __global__ void gla_carry_kernel(GlaArgs a) {
   const int pieces_here = (count + a.piece - 1) / a.piece;
   const size_t row = i / a.value_dim;  // (head, key channel)
   float I = a.state[(size_t)slot * per + i];
-  for (int k = 0; k < pieces_here; ++k) {
-    float* at = a.carried + ((size_t)b * a.pieces + k) * per + i;
-    const bool more = k + 1 < pieces_here;
-    const float E = more ? *at : 0.0f;
-    const float logs = more ? a.decayed[((size_t)b * a.pieces + k) * a.heads * a.key_dim + row] : 0.0f;
-    *at = I;
-    I = fmaf(expf(logs), I, E);
+  for (int k0 = 0; k0 < pieces_here; k0 += 8) {  // eight pieces' ends and decays asked for at once
+    float E[8], logs[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool more = k0 + j + 1 < pieces_here;
+      E[j] = more ? a.carried[((size_t)b * a.pieces + k0 + j) * per + i] : 0.0f;
+      logs[j] = more ? a.decayed[((size_t)b * a.pieces + k0 + j) * a.heads * a.key_dim + row] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (k0 + j < pieces_here) {
+        a.carried[((size_t)b * a.pieces + k0 + j) * per + i] = I;
+        I = fmaf(expf(logs[j]), I, E[j]);
+      }
+    }
   }
 }
 
@@ -560,18 +581,18 @@ extern "C" int nnis_selective_scan(const void* x, int x_dtype, const float* dt_p
   a.x = x; a.x_dtype = x_dtype; a.dt_pre = dt_pre; a.bc = bc; a.z = z; a.z_dtype = z_dtype; a.z_stride = z_stride; a.A = A; a.D = D;
   a.dt_bias = dt_bias; a.state = state; a.seq_slot = seq_slot; a.seq_start = seq_start; a.channels = channels; a.states = states;
   a.y = y; a.y_dtype = y_dtype; a.piece = piece; a.pieces = pieces; a.carried = carried; a.stepped = stepped;
-  const int need = (states + 7) / 8;
+  const int need = (states + 15) / 16;  // lanes of 16 states (of 8 for up to 8 states)
   hipStream_t s = (hipStream_t)stream;
-#define NNIS_SCAN(LANES_, PASS_, PIECES_)                                                                                  \
-  hipLaunchKernelGGL((selective_scan_kernel<LANES_, PASS_>), dim3((channels + 256 / LANES_ - 1) / (256 / LANES_), PIECES_, batch), \
+#define NNIS_SCAN(LANES_, PASS_, PIECES_, PER_)                                                                            \
+  hipLaunchKernelGGL((selective_scan_kernel<LANES_, PASS_, PER_>), dim3((channels + 256 / LANES_ - 1) / (256 / LANES_), PIECES_, batch), \
                      dim3(256), 0, s, a)
-#define NNIS_SCAN_PASS(PASS_, PIECES_)                 \
-  do {                                                 \
-    if (need <= 1) NNIS_SCAN(1, PASS_, PIECES_);       \
-    else if (need <= 2) NNIS_SCAN(2, PASS_, PIECES_);  \
-    else if (need <= 4) NNIS_SCAN(4, PASS_, PIECES_);  \
-    else if (need <= 8) NNIS_SCAN(8, PASS_, PIECES_);  \
-    else NNIS_SCAN(16, PASS_, PIECES_);                \
+#define NNIS_SCAN_PASS(PASS_, PIECES_)                     \
+  do {                                                     \
+    if (states <= 8) NNIS_SCAN(1, PASS_, PIECES_, 8);      \
+    else if (need <= 1) NNIS_SCAN(1, PASS_, PIECES_, 16);  \
+    else if (need <= 2) NNIS_SCAN(2, PASS_, PIECES_, 16);  \
+    else if (need <= 4) NNIS_SCAN(4, PASS_, PIECES_, 16);  \
+    else NNIS_SCAN(8, PASS_, PIECES_, 16);                 \
   } while (0)
   if (pieces <= 1) {
     NNIS_SCAN_PASS(0, 1);

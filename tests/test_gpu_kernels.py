@@ -942,7 +942,7 @@ def test_refusals():
         ops.gemm_ordered(f(3, 8, dtype=torch.float16), f(5, 8), f(3, 5))
     from nnis_amd.errors import Unsupported
 
-    for head_dim in (7, 258, 0):  # a size nobody runs: said as such (the model's check at load raises the same)
+    for head_dim in (258, 0, -2):  # a size nobody runs: said as such (the model's check at load raises the same)
         with pytest.raises(Unsupported, match="head_dim"):
             ops.attention_module(head_dim)
     with pytest.raises(KernelError):

@@ -209,6 +209,45 @@ def test_gated_linear_attention_alone(dtype, heads, dim, vdim, tau, rank, width)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_mixers_side_by_side_and_the_gelu_gate(dtype):
+    """Attention and scan on the same input, each output over its root mean square times its weight, half their sum
+    (the attention's output bias is added by the kernel that norms); the feed-forward with the tanh form of GELU."""
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    width = 72
+    left, right = attention(3, 1, 16, 48, 8, base=300.0, scale=0.4, softcap=5.0), scan(40, 12, 3, 4)
+    rope = build_part("position", {"kind": "rotary_half", "rot_dim": 8, "theta": 300.0, "max_positions": None, "angles": "float64"})
+    rope.bind({}, rt)
+    rope.reach(256)
+    names = dict(q="left.q", k="left.k", v="left.v", o="left.o", q_bias="left.q.b", k_bias="left.k.b", v_bias="left.v.b", o_bias="left.o.b")
+    scan_names = dict(w_in="right.in", conv="right.conv", conv_bias="right.conv.b", w_x="right.x", w_dt="right.dt", dt_bias="right.dt.b",
+                      a_log="right.A_log", d="right.D", w_out="right.o")
+    mixer = build_part("mixer", {
+        "kind": "side_by_side", "width": width, "eps": 1e-4, "weights": ["left.out", "right.out"],
+        "branches": [dict(kind="causal_attention", width=width, heads=3, kv_heads=1, head_dim=16, value_dim=48, scale=0.4, softcap=5.0,
+                          position="r", **names),
+                     dict(kind="selective_scan", width=width, channels=40, states=12, dt_rank=3, taps=4, **scan_names)]},
+        positions={"r": rope})
+    plain_w, part_w = _weights(mixer, dtype, 12, scale={"left.q": 20.0, "left.k": 20.0, "left.o.b": 30.0, "right.in": 20.0, "left.out": 3.0})
+    mixer.bind(part_w, rt)
+    cache = cache_for([mixer.cache_request()], rt, max_tokens=512, max_positions=256)
+    generator = torch.Generator().manual_seed(3)
+    xs = [torch.randn(n, width, generator=generator).to(torch.bfloat16).double() for n in (70, 5)]
+    rnd = Z.identity if dtype == "float32" else Z.bf16_round
+    want = [Z.side_by_side(x, plain_w, {"left": left, "right": right}, 1e-4, rnd) for x in xs]
+    for cuts in ([[70], [5]], [[1, 3, 64, 66, 70], [2, 3, 4, 5]]):
+        got = _run_in_steps(mixer, cache, rt, xs, cuts)
+        for g, w in zip(got, want):
+            _close(g, w, dtype, f"side by side, cuts {cuts[0][:3]}")
+    feed = build_part("feed_forward", {"kind": "gated", "width": width, "inner": 100, "activation": "gelu_tanh", "gate": "gate", "up": "up", "down": "down"})
+    plain_f, part_f = _weights(feed, dtype, 13, scale={"gate": 60.0})
+    feed.bind(part_f, rt)
+    got = feed.forward(xs[0].to(rt.dtype).cuda(), None, rt)
+    _close(got, Z.gated_feed_forward(xs[0], plain_f, rnd), dtype, "feed-forward with the GELU gate")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("streams, width", [(1, 40), (3, 96), (8, 520)])
 def test_streams_and_their_norm(dtype, streams, width):
     """The update of all streams at once from the old ones (mix indexed [from, to]), the weighted sum, the layer norm

@@ -352,7 +352,7 @@ __global__ void selective_scan_carry_kernel(ScanArgs a) {
 //   S <- diag(alpha) S + k v^T
 //   o = S^T (q * scale)
 // A block takes one head of one sequence and a slab of value columns; a thread keeps 16 key rows of one
-// column, the threads of a column (a power of two, up to 16) sit 64 / GROUPS lanes apart in one wave and add
+// column (of two where the head has columns enough), the threads of a column (a power of two, up to 16) sit 64 / GROUPS lanes apart in one wave and add
 // their parts of o by lane exchanges.  Tokens come through LDS a chunk at a time (queries, keys, decays of
 // the head and the slab's values), loaded by the whole block.  o is left raw, in 32-bit.
 // -----------------------------------------------------------------------------
@@ -378,10 +378,12 @@ struct GlaArgs {
 
 // PASS as in selective_scan_kernel: 0 a whole run; 1 a piece from a zero state, leaving its end and the sum of its
 // decays' logarithms; 3 a piece from the state that the carry kernel left for it, writing the outputs.
-template <int GROUPS, int PASS>
+// CPT: value columns a thread keeps (what it reads of queries, keys and decays serves them all)
+template <int GROUPS, int PASS, int CPT>
 __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int kCols = 4 * (kWave / GROUPS);  // value columns of a block (4 waves)
+  constexpr int kSpan = 4 * (kWave / GROUPS);  // columns that the block's threads take side by side (4 waves)
+  constexpr int kCols = CPT * kSpan;           // value columns of a block
   const int b = blockIdx.z / a.pieces, piece = blockIdx.z % a.pieces, head = blockIdx.y;
   const int slot = a.seq_slot[b];
   if (slot < 0) return;
@@ -397,21 +399,28 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
   const int d = a.key_dim, e = a.value_dim;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int group = lane / (kWave / GROUPS);
-  const int col_in_block = wave * (kWave / GROUPS) + lane % (kWave / GROUPS);
-  const int col = blockIdx.x * kCols + col_in_block;
-  const bool live = col < e;
+  const int col_in_span = wave * (kWave / GROUPS) + lane % (kWave / GROUPS);
   float* qs = lds;                    // [chunk][d]
   float* ks = qs + a.chunk * d;       // [chunk][d]
   float* as = ks + a.chunk * d;       // [chunk][d]
   float* vs = as + a.chunk * d;       // [chunk][kCols]
-  float S[16];
-  float* state = a.state + (((size_t)slot * a.heads + head) * d) * e + (live ? col : 0);
-  float* carried = PASS == 0 ? nullptr : a.carried + ((((size_t)b * a.pieces + piece) * a.heads + head) * d) * e + (live ? col : 0);
+  float S[CPT][16];
+  int col[CPT];
+  bool live[CPT];
+  float* state[CPT];
+  float* carried[CPT];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = group * 16 + r;
-    const bool here = live && row < d;
-    S[r] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[(size_t)row * e] : carried[(size_t)row * e]);
+  for (int c = 0; c < CPT; ++c) {
+    col[c] = blockIdx.x * kCols + c * kSpan + col_in_span;
+    live[c] = col[c] < e;
+    state[c] = a.state + (((size_t)slot * a.heads + head) * d) * e + (live[c] ? col[c] : 0);
+    carried[c] = PASS == 0 ? nullptr : a.carried + ((((size_t)b * a.pieces + piece) * a.heads + head) * d) * e + (live[c] ? col[c] : 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = group * 16 + r;
+      const bool here = live[c] && row < d;
+      S[c][r] = !here || PASS == 1 ? 0.0f : (PASS == 0 ? state[c][(size_t)row * e] : carried[c][(size_t)row * e]);
+    }
   }
   float log_sum = 0.0f;  // PASS 1, threads below key_dim of the first slab: the sum of a key channel's log decays
   for (int t0 = first; t0 < last; t0 += a.chunk) {
@@ -432,49 +441,67 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(GlaArgs a) {
     }
     __syncthreads();
     for (int j = 0; j < count; ++j) {
-      const float v = vs[j * kCols + col_in_block];
+      float v[CPT], acc[CPT];
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        v[c] = vs[j * kCols + c * kSpan + col_in_span];
+        acc[c] = 0.0f;
+      }
       const float* qj = qs + j * d + group * 16;
       const float* kj = ks + j * d + group * 16;
       const float* aj = as + j * d + group * 16;
-      float acc = 0.0f;
       if (group * 16 + 16 <= d && d % 4 == 0) {  // whole rows of this group: 16 bytes a read
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const float4 a4 = *(const float4*)(aj + 4 * r4), k4 = *(const float4*)(kj + 4 * r4);
           const float av[4] = {a4.x, a4.y, a4.z, a4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w};
 #pragma unroll
-          for (int i = 0; i < 4; ++i) S[4 * r4 + i] = fmaf(av[i], S[4 * r4 + i], kv[i] * v);
+          for (int c = 0; c < CPT; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) S[c][4 * r4 + i] = fmaf(av[i], S[c][4 * r4 + i], kv[i] * v[c]);
           if (PASS != 1) {
             const float4 q4 = *(const float4*)(qj + 4 * r4);
             const float qv[4] = {q4.x, q4.y, q4.z, q4.w};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc = fmaf(S[4 * r4 + i], qv[i], acc);
+            for (int c = 0; c < CPT; ++c)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) acc[c] = fmaf(S[c][4 * r4 + i], qv[i], acc[c]);
           }
         }
       } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           if (group * 16 + r < d) {
-            S[r] = fmaf(aj[r], S[r], kj[r] * v);
-            if (PASS != 1) acc = fmaf(S[r], qj[r], acc);
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) {
+              S[c][r] = fmaf(aj[r], S[c][r], kj[r] * v[c]);
+              if (PASS != 1) acc[c] = fmaf(S[c][r], qj[r], acc[c]);
+            }
           }
         }
       }
       if (PASS != 1) {
 #pragma unroll
-        for (int offset = kWave / 2; offset >= kWave / GROUPS; offset >>= 1) acc += __shfl_xor(acc, offset, kWave);
-        if (group == 0 && live) a.out[((size_t)(t0 + j) * a.heads + head) * e + col] = acc;
+        for (int c = 0; c < CPT; ++c) {
+#pragma unroll
+          for (int offset = kWave / 2; offset >= kWave / GROUPS; offset >>= 1) acc[c] += __shfl_xor(acc[c], offset, kWave);
+          if (group == 0 && live[c]) a.out[((size_t)(t0 + j) * a.heads + head) * e + col[c]] = acc[c];
+        }
       }
     }
   }
   if (PASS == 1 && blockIdx.x == 0 && (int)threadIdx.x < d)
     a.decayed[(((size_t)b * a.pieces + piece) * a.heads + head) * d + threadIdx.x] = log_sum;
-  if (!live || (PASS == 3 && piece != pieces_here - 1)) return;
-  float* into = PASS == 1 ? carried : state;
+  if (PASS == 3 && piece != pieces_here - 1) return;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = group * 16 + r;
-    if (row < d) into[(size_t)row * e] = S[r];
+  for (int c = 0; c < CPT; ++c) {
+    if (!live[c]) continue;
+    float* into = PASS == 1 ? carried[c] : state[c];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = group * 16 + r;
+      if (row < d) into[(size_t)row * e] = S[c][r];
+    }
   }
 }
 
@@ -627,22 +654,27 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
   a.key_dim = key_dim; a.value_dim = value_dim; a.out = out; a.piece = piece; a.pieces = pieces; a.carried = carried; a.decayed = decayed;
   const int need = (key_dim + 15) / 16;
   const int groups = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : (need <= 8 ? 8 : 16)));
-  const int cols = 4 * (kWave / groups);
+  const int span = 4 * (kWave / groups);
+  const int per_thread = value_dim >= 2 * span ? 2 : 1;  // columns a thread keeps
+  const int cols = per_thread * span;
   int chunk = (int)((40 * 1024) / ((3 * (size_t)key_dim + cols) * sizeof(float)));
   chunk = chunk > 32 ? 32 : (chunk < 1 ? 1 : chunk);
   a.chunk = chunk;
   const size_t lds = (size_t)chunk * (3 * key_dim + cols) * sizeof(float);
   const dim3 grid((value_dim + cols - 1) / cols, heads, batch * pieces);
   hipStream_t s = (hipStream_t)stream;
-#define NNIS_GLA(PASS_)                                                                                   \
-  do {                                                                                                    \
-    switch (groups) {                                                                                     \
-      case 1: hipLaunchKernelGGL((gla_scan_kernel<1, PASS_>), grid, dim3(256), lds, s, a); break;         \
-      case 2: hipLaunchKernelGGL((gla_scan_kernel<2, PASS_>), grid, dim3(256), lds, s, a); break;         \
-      case 4: hipLaunchKernelGGL((gla_scan_kernel<4, PASS_>), grid, dim3(256), lds, s, a); break;         \
-      case 8: hipLaunchKernelGGL((gla_scan_kernel<8, PASS_>), grid, dim3(256), lds, s, a); break;         \
-      default: hipLaunchKernelGGL((gla_scan_kernel<16, PASS_>), grid, dim3(256), lds, s, a); break;       \
-    }                                                                                                     \
+#define NNIS_GLA_CASE(GROUPS_, PASS_)                                                                     \
+  if (per_thread == 2) hipLaunchKernelGGL((gla_scan_kernel<GROUPS_, PASS_, 2>), grid, dim3(256), lds, s, a); \
+  else hipLaunchKernelGGL((gla_scan_kernel<GROUPS_, PASS_, 1>), grid, dim3(256), lds, s, a)
+#define NNIS_GLA(PASS_)                          \
+  do {                                           \
+    switch (groups) {                            \
+      case 1: NNIS_GLA_CASE(1, PASS_); break;    \
+      case 2: NNIS_GLA_CASE(2, PASS_); break;    \
+      case 4: NNIS_GLA_CASE(4, PASS_); break;    \
+      case 8: NNIS_GLA_CASE(8, PASS_); break;    \
+      default: NNIS_GLA_CASE(16, PASS_); break;  \
+    }                                            \
   } while (0)
   if (pieces <= 1) {
     NNIS_GLA(0);
@@ -653,6 +685,7 @@ extern "C" int nnis_gla_scan(const void* q, const void* k, const void* v, int qk
     NNIS_GLA(3);
   }
 #undef NNIS_GLA
+#undef NNIS_GLA_CASE
   NNIS_LAUNCH_CHECK("gla_scan");
   return 0;
 }

@@ -176,7 +176,10 @@ def test_selective_scan_alone(dtype, channels, states, dt_rank, taps, width):
     assert float(want[0][-1].abs().max()) > 1e-3
     # the state carries far: dropping the first token changes the last output
     assert _relative(Z.selective_scan(xs[0][1:], plain_w, sizes)[-1], Z.selective_scan(xs[0], plain_w, sizes)[-1]) > 1e-4
-    for cuts in ([[90], [1], [17]], [[1, 2, 3, 5, 6, 64, 66, 88, 89, 90], [1], [2, 4, 5, 6, 7, 17]], [list(range(1, 91)), [1], list(range(1, 18))]):
+    # (the kernels cut a run of 48 tokens or more into pieces of 16 or more that run side by side: runs just below and at
+    # that length, and pieces that end inside a run's last tokens)
+    for cuts in ([[90], [1], [17]], [[1, 2, 3, 5, 6, 64, 66, 88, 89, 90], [1], [2, 4, 5, 6, 7, 17]], [list(range(1, 91)), [1], list(range(1, 18))],
+                 [[47, 90], [1], [17]], [[48, 90], [1], [16, 17]], [[41, 90], [1], [17]]):
         got = _run_in_steps(mixer, cache, rt, xs, cuts)
         for g, w, n in zip(got, want, lengths):
             _close(g, w, dtype, f"scan length {n} in {len(cuts[0])} steps")
@@ -202,7 +205,8 @@ def test_gated_linear_attention_alone(dtype, heads, dim, vdim, tau, rank, width)
     want = [Z.gated_linear_attention(x, plain_w, sizes, 1e-5, Z.identity if dtype == "float32" else Z.bf16_round) for x in xs]
     if tau >= 4.0:  # the first token is still in the state
         assert _relative(Z.gated_linear_attention(xs[0][1:], plain_w, sizes, 1e-5)[-1], Z.gated_linear_attention(xs[0], plain_w, sizes, 1e-5)[-1]) > 1e-3
-    for cuts in ([[100], [2], [33]], [[2, 4, 31, 32, 33, 64, 65, 98, 100], [1, 2], [3, 33]], [list(range(1, 101)), [1, 2], list(range(1, 34))]):
+    for cuts in ([[100], [2], [33]], [[2, 4, 31, 32, 33, 64, 65, 98, 100], [1, 2], [3, 33]], [list(range(1, 101)), [1, 2], list(range(1, 34))],
+                 [[47, 100], [2], [33]], [[48, 100], [2], [32, 33]], [[51, 100], [2], [33]]):  # (runs around the length from which they are cut into pieces)
         got = _run_in_steps(mixer, cache, rt, xs, cuts)
         for g, w, n in zip(got, want, lengths):
             _close(g, w, dtype, f"gated linear attention length {n} in {len(cuts[0])} steps")

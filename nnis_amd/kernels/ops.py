@@ -523,8 +523,31 @@ _gemm_workspaces = {}
 PAIR_COUNTS = 1024  # 32-bit words kept behind the workspace for the strips' counts
 
 
+# Work that runs beside the main stream's (the branches of mixers side by side, on a second stream) has scratch
+# of its own: a lane names whose.  Lane 0 is everybody's unless a part says otherwise around its launches.
+_lane = 0
+
+
+class lane:
+    """``with ops.lane(1): ...``: the launches inside take lane 1's scratch (the products' workspace), so that they
+    may run at the same time as launches outside that share the device."""
+
+    def __init__(self, number: int):
+        self.number, self.before = int(number), 0
+
+    def __enter__(self):
+        global _lane
+        self.before, _lane = _lane, self.number
+        return self
+
+    def __exit__(self, *exc):
+        global _lane
+        _lane = self.before
+        return False
+
+
 def _gemm_workspace(device) -> Optional[torch.Tensor]:
-    key = (device.type, device.index)
+    key = (device.type, device.index, _lane)
     held = _gemm_workspaces.get(key)
     if held is None and not torch.cuda.is_current_stream_capturing():
         # behind the workspace proper: the counts of the strips that two blocks share (`gemm_residual`), zero between calls

@@ -53,8 +53,8 @@ ZIF_C = zifunex(
     layers=[
         parallel(attention(6, 1, 48, 64, 24, base=100000.0, scale=0.1443, softcap=15.0), scan(96, 16, 6, 4), ff=200),
         gla(heads=1, dim=64, vdim=128, tau=32.0, rank=24, ff=144),
-        parallel(attention(2, 2, 64, 32, 64, base=10000.0, scale=0.125, softcap=30.0), scan(160, 24, 10, 4)),
-        gla(heads=4, dim=32, vdim=32, tau=16.0, rank=8),
+        parallel(attention(2, 2, 64, 32, 64, base=10000.0, scale=0.13, softcap=28.0), scan(160, 20, 10, 4)),
+        gla(heads=5, dim=24, vdim=40, tau=12.0, rank=8),
     ],
     loop=(1, 3, 3))
 

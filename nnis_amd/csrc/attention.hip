@@ -66,6 +66,11 @@ struct AttnArgs {
   int window;  // 0: all keys
   float scale;
   float softcap;  // 0: none; else a score s becomes softcap * tanh(s / softcap)
+  // Beyond the plain formula, each off when zero or null:
+  int keep_first;      // with a window: keys at positions below this stay visible to every later query
+  const float* bias;   // [heads, reach + 1]: added to the scaled score of a key `n` positions back, row min(n, reach)
+  int reach;
+  const float* sink;   // [heads]: a score that joins the softmax's denominator and has no value
 };
 
 // One wave per (token, query head); lanes take keys lo+lane, lo+lane+64, ...,
@@ -104,8 +109,9 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   float o[HDV];
 #pragma unroll
   for (int d = 0; d < HDV; ++d) o[d] = 0.0f;
+  const float* bias_row = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
 
-  for (int j = lo + lane; j < kv_len; j += kWave) {
+  auto take = [&](int j) {
     const int page = pages[j / kPageTokens];
     const int r = j % kPageTokens;
     const CacheT* keys = kp + ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(HD);
@@ -114,6 +120,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
     for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_f32(keys[nnis_k_offset(r, d)]), dot);
     float s = dot * a.scale;
     if (a.softcap > 0.0f) s = a.softcap * tanhf(s / a.softcap);
+    if (bias_row) s += bias_row[min(pos - j, a.reach)];
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first key
     const float p = expf(s - m_new);
@@ -122,11 +129,16 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
 #pragma unroll
     for (int d = 0; d < HDV; ++d) o[d] = o[d] * alpha + p * to_f32(values[nnis_v_offset(d, r)]);
     m = m_new;
-  }
+  };
+  const int kept = min(a.keep_first, lo);  // the kept first keys that the window has left behind
+  for (int j = lane; j < kept; j += kWave) take(j);
+  for (int j = lo + lane; j < kv_len; j += kWave) take(j);
 
-  const float m_all = wave_max(m);
+  float m_all = wave_max(m);
+  const float sink = a.sink ? a.sink[head] : -INFINITY;
+  m_all = fmaxf(m_all, sink);
   const float factor = (m == -INFINITY) ? 0.0f : expf(m - m_all);
-  const float l_all = wave_sum(l * factor);
+  const float l_all = wave_sum(l * factor) + (a.sink ? expf(sink - m_all) : 0.0f);
   const float inv = 1.0f / l_all;
   float mine[(HDV + kWave - 1) / kWave];
 #pragma unroll
@@ -1156,10 +1168,11 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
 
 }  // namespace
 
-extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
+extern "C" int nnis_attention_rows_more(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
                                    const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
                                    const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
-                                   int head_dim, int window, float scale, int value_dim, float softcap, void* stream) {
+                                   int head_dim, int window, float scale, int value_dim, float softcap, int keep_first,
+                                        const float* bias, int reach, const float* sink, void* stream) {
   NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
   NNIS_REQUIRE((value_dim <= 0 ? head_dim : value_dim) == HDV, "attention: this module is compiled for values of %d channels, got %d", HDV, value_dim);
   NNIS_REQUIRE(softcap >= 0.0f, "attention: the cap of the scores must not be negative, got %g", (double)softcap);
@@ -1168,12 +1181,14 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
   NNIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: %d heads do not divide into %d kv heads",
                heads, kv_heads);
   NNIS_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window %d or block table width %d", window, max_pages);
+  NNIS_REQUIRE(keep_first >= 0 && (bias == nullptr || reach >= 0), "attention: bad keep_first %d or reach %d", keep_first, reach);
   if (tokens <= 0) return 0;
   AttnArgs a;
   a.q = q; a.q_dtype = q_dtype; a.out = out; a.out_dtype = out_dtype;
   a.k_pages = k_pages; a.v_pages = v_pages; a.cache_dtype = cache_dtype;
   a.block_table = block_table; a.max_pages = max_pages; a.tok_slot = tok_slot; a.tok_pos = tok_pos;
   a.tokens = tokens; a.heads = heads; a.kv_heads = kv_heads; a.window = window; a.scale = scale; a.softcap = softcap;
+  a.keep_first = window > 0 ? keep_first : 0; a.bias = bias; a.reach = reach; a.sink = sink;
   const long long items = (long long)tokens * heads;
   const unsigned blocks = (unsigned)((items + 3) / 4);
   if (cache_dtype == NNIS_F32) {
@@ -1183,6 +1198,16 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
   }
   NNIS_LAUNCH_CHECK("attention_rows");
   return 0;
+}
+
+
+extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
+                                   const void* v_pages, int cache_dtype, const int* block_table, int max_pages,
+                                   const int* tok_slot, const int* tok_pos, int tokens, int heads, int kv_heads,
+                                   int head_dim, int window, float scale, int value_dim, float softcap, void* stream) {
+  return nnis_attention_rows_more(q, q_dtype, out, out_dtype, k_pages, v_pages, cache_dtype, block_table, max_pages, tok_slot,
+                                  tok_pos, tokens, heads, kv_heads, head_dim, window, scale, value_dim, softcap, 0, nullptr, 0,
+                                  nullptr, stream);
 }
 
 

@@ -13,11 +13,11 @@ thread_local char g_nnis_error[512] = {0};
 extern "C" const char* nnis_last_error() { return g_nnis_error; }
 
 // -----------------------------------------------------------------------------
-// embedding: out[t, :] = table[ids[t], :]   (a row copy, no scaling;
-// /root/reference/crates/nnis-kernels/src/gather.rs:17-33)
+// embedding: out[t, :] = table[ids[t], :] * scale   (a row copy, /root/reference/crates/nnis-kernels/src/gather.rs:17-33;
+// the scale is 1 for a model that has none: the product is then exact)
 // -----------------------------------------------------------------------------
 __global__ void embed_kernel(const int* __restrict__ ids, const void* __restrict__ table, int table_dtype,
-                             float* __restrict__ out, int width, int vocab) {
+                             float* __restrict__ out, int width, int vocab, float scale) {
   const int token = blockIdx.x;
   const int id = ids[token];
   float* dst = out + (size_t)token * width;
@@ -26,16 +26,16 @@ __global__ void embed_kernel(const int* __restrict__ ids, const void* __restrict
     return;
   }
   const size_t base = (size_t)id * width;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_as_f32(table, table_dtype, base + c);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_as_f32(table, table_dtype, base + c) * scale;
 }
 
 extern "C" int nnis_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
-                          int vocab, void* stream) {
+                          int vocab, float scale, void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(table_dtype), "embed: unknown table dtype %d", table_dtype);
   NNIS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes tokens=%d width=%d vocab=%d", tokens, width, vocab);
   if (tokens == 0) return 0;
   hipLaunchKernelGGL(embed_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, ids, table, table_dtype, out,
-                     width, vocab);
+                     width, vocab, scale);
   NNIS_LAUNCH_CHECK("embed");
   return 0;
 }
@@ -44,7 +44,7 @@ extern "C" int nnis_embed(const int* ids, const void* table, int table_dtype, fl
 // that shares the table needs that order, and the table is then kept once.  8 consecutive channels of a row lie
 // together (16 bytes); a thread copies one such piece.
 __global__ void embed_packed_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ packed,
-                                    float* __restrict__ out, int width, int vocab) {
+                                    float* __restrict__ out, int width, int vocab, float scale) {
   const int token = blockIdx.x;
   const int id = ids[token];
   float* dst = out + (size_t)token * width;
@@ -60,19 +60,19 @@ __global__ void embed_packed_kernel(const int* __restrict__ ids, const bf16_t* _
     const uint32_t words[4] = {piece.x, piece.y, piece.z, piece.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {  // bfloat16 widens by a shift
-      dst[k + 2 * i] = __uint_as_float(words[i] << 16);
-      dst[k + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
+      dst[k + 2 * i] = __uint_as_float(words[i] << 16) * scale;
+      dst[k + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u) * scale;
     }
   }
 }
 
 extern "C" int nnis_embed_packed(const int* ids, const void* packed, float* out, int tokens, int width, int vocab,
-                                 void* stream) {
+                                 float scale, void* stream) {
   NNIS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes tokens=%d width=%d vocab=%d", tokens, width, vocab);
   NNIS_REQUIRE(width % 8 == 0, "embed: a packed table has a width that is a multiple of 8, got %d", width);
   if (tokens == 0) return 0;
   hipLaunchKernelGGL(embed_packed_kernel, dim3(tokens), dim3(64 * ((width / 8 + 63) / 64 > 4 ? 4 : (width / 8 + 63) / 64)), 0,
-                     (hipStream_t)stream, ids, (const bf16_t*)packed, out, width, vocab);
+                     (hipStream_t)stream, ids, (const bf16_t*)packed, out, width, vocab, scale);
   NNIS_LAUNCH_CHECK("embed_packed");
   return 0;
 }

@@ -1,0 +1,170 @@
+// Row-wise kernels of attention over a cached latent: every token keeps one normed vector c (and, where the
+// mixer rotates, one rotated key part shared by all heads) instead of keys and values per head.  With the
+// heads' key and value maps folded into the query and output projections, the latent is key and value of one
+// shared key/value head: keys [c, rotated part], values c.  What is left between the projections is here:
+//   latent_prepare   from one fused projection's row [query latent | c | rotated key part | gate logits]:
+//                    the query latent divided by its root mean square and weighted; c likewise, written with
+//                    the rotated key part into the token's page of keys and, alone, into its page of values;
+//                    the gates as sigmoid(logit)
+//   latent_rotate_q  the rotated channels of every head's query, in place
+//   head_scale       a head's output multiplied by its gate, in place
+// A rotation pairs channel 2i with channel 2i + 1: (u, v) -> (u cos a - v sin a, v cos a + u sin a), a =
+// position * frequency i, cosines and sines from tables [positions, pairs] made on the host.  Norms, angles,
+// rotations and gates are 32-bit; storage types are chosen at run time.
+#include "common.h"
+
+thread_local char g_nnis_error[512] = {0};
+extern "C" const char* nnis_last_error() { return g_nnis_error; }
+
+namespace {
+
+struct PrepareArgs {
+  const void* proj;  // [tokens, q_rank + kv_rank + rot_dim + gates]
+  int proj_dtype;
+  int q_rank, kv_rank, rot_dim, gates;
+  const void* q_weight;  // [q_rank]
+  const void* c_weight;  // [kv_rank]
+  int w_dtype;
+  float eps;
+  const float* cos_table;  // [positions, rot_dim / 2]
+  const float* sin_table;
+  int positions;
+  const int* tok_slot;
+  const int* tok_pos;
+  void* cq;  // [tokens, q_rank]
+  int cq_dtype;
+  void* k_pages;  // one key/value head: keys of kv_rank + rot_dim channels, values of kv_rank
+  void* v_pages;
+  int cache_dtype;
+  const int* block_table;
+  int max_pages;
+  float* gate;  // [tokens, gates]
+};
+
+__global__ __launch_bounds__(256) void latent_prepare_kernel(PrepareArgs a) {
+  __shared__ float scratch[16];
+  const int token = blockIdx.x;
+  const int row_width = a.q_rank + a.kv_rank + a.rot_dim + a.gates;
+  const size_t row = (size_t)token * row_width;
+  float ss_q = 0.0f, ss_c = 0.0f;
+  for (int i = threadIdx.x; i < a.q_rank; i += blockDim.x) {
+    const float v = load_as_f32(a.proj, a.proj_dtype, row + i);
+    ss_q = fmaf(v, v, ss_q);
+  }
+  for (int i = threadIdx.x; i < a.kv_rank; i += blockDim.x) {
+    const float v = load_as_f32(a.proj, a.proj_dtype, row + a.q_rank + i);
+    ss_c = fmaf(v, v, ss_c);
+  }
+  const float inv_q = a.q_rank > 0 ? 1.0f / sqrtf(block_sum(ss_q, scratch) / (float)a.q_rank + a.eps) : 0.0f;
+  const float inv_c = 1.0f / sqrtf(block_sum(ss_c, scratch) / (float)a.kv_rank + a.eps);
+  for (int i = threadIdx.x; i < a.q_rank; i += blockDim.x)
+    store_from_f32(a.cq, a.cq_dtype, (size_t)token * a.q_rank + i,
+                   load_as_f32(a.proj, a.proj_dtype, row + i) * inv_q * load_as_f32(a.q_weight, a.w_dtype, i));
+  for (int i = threadIdx.x; i < a.gates; i += blockDim.x) {
+    const float g = load_as_f32(a.proj, a.proj_dtype, row + a.q_rank + a.kv_rank + a.rot_dim + i);
+    a.gate[(size_t)token * a.gates + i] = 1.0f / (1.0f + expf(-g));
+  }
+  const int slot = a.tok_slot[token];
+  if (slot < 0 || a.k_pages == nullptr) return;  // a padding row, or a run that keeps no cache of its own
+  const int pos = a.tok_pos[token];
+  const int page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+  const int at = pos % kPageTokens;
+  const size_t k_base = (size_t)page * nnis_k_page_elems(a.kv_rank + a.rot_dim);
+  const size_t v_base = (size_t)page * nnis_v_page_elems(a.kv_rank);
+  for (int i = threadIdx.x; i < a.kv_rank; i += blockDim.x) {
+    const float c = load_as_f32(a.proj, a.proj_dtype, row + a.q_rank + i) * inv_c * load_as_f32(a.c_weight, a.w_dtype, i);
+    store_from_f32(a.k_pages, a.cache_dtype, k_base + nnis_k_offset(at, i), c);
+    store_from_f32(a.v_pages, a.cache_dtype, v_base + nnis_v_offset(i, at), c);
+  }
+  const int pairs = a.rot_dim / 2;
+  const int table_row = pos < a.positions ? pos : a.positions - 1;  // (the engine refuses a step beyond the tables before it launches)
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const float u = load_as_f32(a.proj, a.proj_dtype, row + a.q_rank + a.kv_rank + 2 * i);
+    const float v = load_as_f32(a.proj, a.proj_dtype, row + a.q_rank + a.kv_rank + 2 * i + 1);
+    const float c = a.cos_table[(size_t)table_row * pairs + i], s = a.sin_table[(size_t)table_row * pairs + i];
+    store_from_f32(a.k_pages, a.cache_dtype, k_base + nnis_k_offset(at, a.kv_rank + 2 * i), u * c - v * s);
+    store_from_f32(a.k_pages, a.cache_dtype, k_base + nnis_k_offset(at, a.kv_rank + 2 * i + 1), v * c + u * s);
+  }
+}
+
+__global__ void latent_rotate_q_kernel(void* __restrict__ q, int q_dtype, int heads, int head_width, int first, int pairs,
+                                       const float* __restrict__ cos_table, const float* __restrict__ sin_table, int positions,
+                                       const int* __restrict__ tok_pos, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int pair = (int)(i % pairs);
+    const size_t head_row = i / pairs;  // token * heads + head
+    const int token = (int)(head_row / heads);
+    int pos = tok_pos[token];
+    pos = pos < 0 ? 0 : (pos < positions ? pos : positions - 1);
+    const size_t at = head_row * head_width + first + 2 * pair;
+    const float u = load_as_f32(q, q_dtype, at), v = load_as_f32(q, q_dtype, at + 1);
+    const float c = cos_table[(size_t)pos * pairs + pair], s = sin_table[(size_t)pos * pairs + pair];
+    store_from_f32(q, q_dtype, at, u * c - v * s);
+    store_from_f32(q, q_dtype, at + 1, v * c + u * s);
+  }
+}
+
+__global__ void head_scale_kernel(void* __restrict__ o, int o_dtype, const float* __restrict__ gate, int channels, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    store_from_f32(o, o_dtype, i, load_as_f32(o, o_dtype, i) * gate[i / channels]);
+}
+
+unsigned blocks_for(size_t total) {
+  size_t blocks = (total + 255) / 256;
+  return (unsigned)(blocks > 65536 ? 65536 : blocks);
+}
+
+}  // namespace
+
+extern "C" int nnis_latent_prepare(const void* proj, int proj_dtype, int tokens, int q_rank, int kv_rank, int rot_dim, int gates,
+                                   const void* q_weight, const void* c_weight, int w_dtype, float eps, const float* cos_table,
+                                   const float* sin_table, int positions, const int* tok_slot, const int* tok_pos, void* cq,
+                                   int cq_dtype, void* k_pages, void* v_pages, int cache_dtype, const int* block_table,
+                                   int max_pages, float* gate, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(proj_dtype) && nnis_dtype_ok(w_dtype) && nnis_dtype_ok(cq_dtype) && nnis_dtype_ok(cache_dtype),
+               "latent_prepare: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && q_rank >= 0 && kv_rank > 0 && rot_dim >= 0 && rot_dim % 2 == 0 && gates >= 0,
+               "latent_prepare: bad sizes (q_rank %d, kv_rank %d, rot_dim %d, gates %d)", q_rank, kv_rank, rot_dim, gates);
+  NNIS_REQUIRE(proj && c_weight && tok_slot && tok_pos && eps > 0.0f, "latent_prepare: missing operands");
+  NNIS_REQUIRE(q_rank == 0 || (q_weight && cq), "latent_prepare: a query latent needs its weight and its output");
+  NNIS_REQUIRE(rot_dim == 0 || (cos_table && sin_table && positions > 0), "latent_prepare: a rotation needs its tables");
+  NNIS_REQUIRE(gates == 0 || gate, "latent_prepare: gates need their output");
+  NNIS_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || (block_table && max_pages > 0)),
+               "latent_prepare: pages come with values and a block table");
+  if (tokens == 0) return 0;
+  PrepareArgs a;
+  a.proj = proj; a.proj_dtype = proj_dtype; a.q_rank = q_rank; a.kv_rank = kv_rank; a.rot_dim = rot_dim; a.gates = gates;
+  a.q_weight = q_weight; a.c_weight = c_weight; a.w_dtype = w_dtype; a.eps = eps; a.cos_table = cos_table; a.sin_table = sin_table;
+  a.positions = positions; a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.cq = cq; a.cq_dtype = cq_dtype; a.k_pages = k_pages;
+  a.v_pages = v_pages; a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages; a.gate = gate;
+  const int widest = q_rank > kv_rank ? q_rank : kv_rank;
+  const int threads = widest >= 256 ? 256 : (widest >= 128 ? 128 : 64);
+  hipLaunchKernelGGL(latent_prepare_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("latent_prepare");
+  return 0;
+}
+
+extern "C" int nnis_latent_rotate_q(void* q, int q_dtype, int tokens, int heads, int head_width, int first, int rot_dim,
+                                    const float* cos_table, const float* sin_table, int positions, const int* tok_pos,
+                                    void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(q_dtype), "latent_rotate_q: unknown dtype");
+  NNIS_REQUIRE(q && cos_table && sin_table && tok_pos && positions > 0, "latent_rotate_q: missing operands");
+  NNIS_REQUIRE(tokens >= 0 && heads > 0 && rot_dim > 0 && rot_dim % 2 == 0 && first >= 0 && first + rot_dim <= head_width,
+               "latent_rotate_q: %d rotated channels from %d on do not fit heads of %d", rot_dim, first, head_width);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * heads * (rot_dim / 2);
+  hipLaunchKernelGGL(latent_rotate_q_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, q, q_dtype, heads,
+                     head_width, first, rot_dim / 2, cos_table, sin_table, positions, tok_pos, total);
+  NNIS_LAUNCH_CHECK("latent_rotate_q");
+  return 0;
+}
+
+extern "C" int nnis_head_scale(void* o, int o_dtype, const float* gate, int tokens, int heads, int channels, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(o_dtype), "head_scale: unknown dtype");
+  NNIS_REQUIRE(o && gate && tokens >= 0 && heads > 0 && channels > 0, "head_scale: bad arguments");
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * heads * channels;
+  hipLaunchKernelGGL(head_scale_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, o, o_dtype, gate, channels, total);
+  NNIS_LAUNCH_CHECK("head_scale");
+  return 0;
+}

@@ -411,9 +411,11 @@ extern "C" int nnis_branch_mean(const void* const* y, const void* const* weight,
 // Gated activation on a fused [tokens, 2 * inner] projection (gate columns first): out = act(gate) * up.
 //   act 0: SiLU, gate / (1 + exp(-gate))
 //   act 1: the tanh form of GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
+//   act 2: ReLU, max(g, 0)
 // -----------------------------------------------------------------------------
 __device__ __forceinline__ float gate_activation(float g, int act) {
   if (act == 0) return g / (1.0f + expf(-g));
+  if (act == 2) return fmaxf(g, 0.0f);
   const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
   return 0.5f * g * (1.0f + tanhf(inner));
 }
@@ -449,7 +451,7 @@ extern "C" int nnis_gated_act(const void* gate_up, int in_dtype, void* out, int 
                               void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(in_dtype) && nnis_dtype_ok(out_dtype), "gated_act: unknown dtype");
   NNIS_REQUIRE(tokens >= 0 && inner > 0, "gated_act: bad sizes tokens=%d inner=%d", tokens, inner);
-  NNIS_REQUIRE(act == 0 || act == 1, "gated_act: unknown activation %d", act);
+  NNIS_REQUIRE(act >= 0 && act <= 2, "gated_act: unknown activation %d", act);
   if (tokens == 0) return 0;
   if (in_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && inner % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)out % 16 == 0) {
     const size_t groups = (size_t)tokens * (inner / 8);
@@ -488,5 +490,99 @@ extern "C" int nnis_add_bias(void* y, int y_dtype, const void* bias, int bias_dt
   hipLaunchKernelGGL(add_bias_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, y, y_dtype, bias, bias_dtype, width,
                      total);
   NNIS_LAUNCH_CHECK("add_bias");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// The residual stream's step around a norm without statistics, y -> tanh(alpha y) * w + b (alpha a scalar, w and
+// b per channel; nothing of a row is summed, so any cut of a row into threads will do).  One kernel does what
+// lies between two projections of a layer that norms its sublayers before and after:
+//   v = x[src]                                       the stream, 32-bit (0 without one)
+//   v += post ? tanh(post_alpha y) post_w + post_b : y     a sublayer's output, normed on its way in (if y)
+//   v += rows_add[src]                                a second stream of rows (the embedding, on re-entry)
+//   v += vec_add                                      a vector per channel
+//   x_out[src] = v                                    (without a row list; x_out may be x itself)
+//   h[r] = next ? tanh(next_alpha v) next_w + next_b : v   the input of what comes next (if h)
+// src = rows ? rows[r] : r.  All arithmetic in 32-bit; y, the weights and h in the type their codes say.
+// -----------------------------------------------------------------------------
+struct TanhNormArgs {
+  const float* x;
+  float* x_out;
+  const void* y;
+  int y_dtype;
+  const void* post_w;
+  const void* post_b;
+  float post_alpha;
+  const float* rows_add;
+  const void* vec_add;
+  const void* next_w;
+  const void* next_b;
+  float next_alpha;
+  int w_dtype;
+  void* h;
+  int h_dtype;
+  const int* rows;
+  int width;
+  size_t total;  // output rows x width
+};
+
+__global__ void tanh_norm_step_kernel(TanhNormArgs a) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = i / a.width;
+    const int c = (int)(i % a.width);
+    const size_t src = (a.rows ? (size_t)a.rows[r] : r) * a.width + c;
+    float v = a.x ? a.x[src] : 0.0f;
+    if (a.y) {
+      float y = load_as_f32(a.y, a.y_dtype, src);
+      if (a.post_w) y = tanhf(a.post_alpha * y) * load_as_f32(a.post_w, a.w_dtype, c) + load_as_f32(a.post_b, a.w_dtype, c);
+      v += y;
+    }
+    if (a.rows_add) v += a.rows_add[src];
+    if (a.vec_add) v += load_as_f32(a.vec_add, a.w_dtype, c);
+    if (a.x_out) a.x_out[src] = v;
+    if (a.h) {
+      const float h = a.next_w ? tanhf(a.next_alpha * v) * load_as_f32(a.next_w, a.w_dtype, c) + load_as_f32(a.next_b, a.w_dtype, c) : v;
+      store_from_f32(a.h, a.h_dtype, i, h);
+    }
+  }
+}
+
+extern "C" int nnis_tanh_norm_step(const float* x, float* x_out, const void* y, int y_dtype, const void* post_w, const void* post_b,
+                                   float post_alpha, const float* rows_add, const void* vec_add, const void* next_w,
+                                   const void* next_b, float next_alpha, int w_dtype, void* h, int h_dtype, const int* rows,
+                                   int out_rows, int width, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(y_dtype) && nnis_dtype_ok(w_dtype) && nnis_dtype_ok(h_dtype), "tanh_norm_step: unknown dtype");
+  NNIS_REQUIRE((x || y) && out_rows >= 0 && width > 0, "tanh_norm_step: bad arguments (rows %d, width %d)", out_rows, width);
+  NNIS_REQUIRE((post_w == nullptr) == (post_b == nullptr) && (next_w == nullptr) == (next_b == nullptr),
+               "tanh_norm_step: a norm comes with its weight and its bias");
+  NNIS_REQUIRE(!(rows && x_out), "tanh_norm_step: a step over a list of rows leaves the stream as it is");
+  NNIS_REQUIRE(x_out || h, "tanh_norm_step: nothing to write");
+  if (out_rows == 0) return 0;
+  TanhNormArgs a;
+  a.x = x; a.x_out = x_out; a.y = y; a.y_dtype = y_dtype; a.post_w = post_w; a.post_b = post_b; a.post_alpha = post_alpha;
+  a.rows_add = rows_add; a.vec_add = vec_add; a.next_w = next_w; a.next_b = next_b; a.next_alpha = next_alpha; a.w_dtype = w_dtype;
+  a.h = h; a.h_dtype = h_dtype; a.rows = rows; a.width = width; a.total = (size_t)out_rows * width;
+  size_t blocks = (a.total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(tanh_norm_step_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("tanh_norm_step");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// Logits bent by a cap, in place: x -> cap * tanh(x / cap)   (32-bit rows)
+// -----------------------------------------------------------------------------
+__global__ void tanh_cap_kernel(float* __restrict__ x, float cap, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int nnis_tanh_cap(float* x, float cap, long long total, void* stream) {
+  NNIS_REQUIRE(x && cap > 0.0f && total >= 0, "tanh_cap: bad arguments (cap %g)", (double)cap);
+  if (total == 0) return 0;
+  size_t blocks = ((size_t)total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(tanh_cap_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, cap, (size_t)total);
+  NNIS_LAUNCH_CHECK("tanh_cap");
   return 0;
 }

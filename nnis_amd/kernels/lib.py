@@ -124,6 +124,8 @@ register_module("core", ["elementwise.hip", "residual.hip", "gemm.hip", "gemm_mf
 register_module_family("attn_hd", _attention_recipe)
 # the mixers that carry a state of fixed size (convolution, selective scan, gated linear attention)
 register_module("recurrent", ["recurrent.hip"], headers=["common.h"])
+# attention over a cached latent: what lies between its projections (norms of the latents, rotation, cache write, gates)
+register_module("latent", ["latent.hip"], headers=["common.h"])
 # plain host references of the kernels' operations, for the tests (no device code: the host compiler builds them)
 register_module("reference", ["reference.cpp"], host_only=True)
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off"]  # a multiply-add is fused only where the source says fmaf
@@ -297,7 +299,7 @@ def load_module(module: str, build_if_missing: bool = True) -> ctypes.CDLL:
 
 
 def all_prebuilt_modules() -> List[str]:
-    return ["core", "reference", "recurrent"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS] + list(PREBUILT_WIDE_VALUES)
+    return ["core", "reference", "recurrent", "latent"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS] + list(PREBUILT_WIDE_VALUES)
 
 
 def build_all(force: bool = True, jobs: int = 4) -> List[str]:

@@ -24,8 +24,8 @@ _U64 = ctypes.c_uint64
 _I64 = ctypes.c_longlong
 
 _CORE_SIGNATURES = {
-    "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
-    "nnis_embed_packed": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _FLT, _VOID],
+    "nnis_embed_packed": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _FLT, _VOID],
     "nnis_step_tables": [_VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID],
     "nnis_rmsnorm": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
@@ -39,6 +39,9 @@ _CORE_SIGNATURES = {
     "nnis_branch_mean": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT, _VOID, _INT, _VOID],
     "nnis_gated_act": [_VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_add_bias": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_tanh_norm_step": [_VOID, _VOID, _VOID, _INT, _VOID, _VOID, _FLT, _VOID, _VOID, _VOID, _VOID, _FLT, _INT, _VOID, _INT, _VOID,
+                            _INT, _INT, _VOID],
+    "nnis_tanh_cap": [_VOID, _FLT, _I64, _VOID],
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID, _VOID],
     "nnis_argmax_scratch": [_INT, _INT],
     "nnis_argmax_static": [_VOID, _VOID, _INT, _INT, _VOID],
@@ -61,6 +64,8 @@ _CORE_SIGNATURES = {
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
                             _INT, _INT, _FLT, _INT, _FLT, _VOID],
+    "nnis_attention_rows_more": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
+                                 _INT, _INT, _FLT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _VOID],
@@ -80,6 +85,13 @@ _RECURRENT_SIGNATURES = {
                       _VOID, _INT, _INT, _VOID, _VOID, _VOID],
     "nnis_gla_decays": [_VOID, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_head_norm_gate": [_VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _FLT, _VOID],
+}
+
+_LATENT_SIGNATURES = {
+    "nnis_latent_prepare": [_VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _INT, _FLT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID,
+                            _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID],
+    "nnis_latent_rotate_q": [_VOID, _INT, _INT, _INT, _INT, _INT, _INT, _VOID, _VOID, _INT, _VOID, _VOID],
+    "nnis_head_scale": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
 }
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -139,6 +151,17 @@ def recurrent():
     if _recurrent is None:
         _recurrent = _bind("recurrent", _RECURRENT_SIGNATURES)
     return _recurrent
+
+
+_latent = None
+
+
+def latent():
+    """The module of attention over a cached latent (norms of the latents, rotation, cache write, gates)."""
+    global _latent
+    if _latent is None:
+        _latent = _bind("latent", _LATENT_SIGNATURES)
+    return _latent
 
 
 def core():
@@ -221,8 +244,8 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 # ---------------------------------------------------------------------------
 
-def embed(ids: torch.Tensor, table, out: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :] widened to 32-bit; ids outside the table give a zero row.
+def embed(ids: torch.Tensor, table, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] widened to 32-bit, times ``scale``; ids outside the table give a zero row.
     ``table``: a matrix [vocab, width], or the ``PackedWeight`` of one (a table that a head shares)."""
     _dev(ids, "ids"), _dev(table, "embedding table"), _dev(out, "out")
     tokens, width = out.shape
@@ -232,13 +255,13 @@ def embed(ids: torch.Tensor, table, out: torch.Tensor) -> torch.Tensor:
         if table.shape[1] != width or out.dtype != torch.float32:
             raise KernelError(f"embed: packed table {table.shape} / out {tuple(out.shape)} {out.dtype} do not fit")
         lib = core()
-        _check(lib, lib.nnis_embed_packed(ids.data_ptr(), table.data_ptr(), out.data_ptr(), tokens, width, table.shape[0], _stream()))
+        _check(lib, lib.nnis_embed_packed(ids.data_ptr(), table.data_ptr(), out.data_ptr(), tokens, width, table.shape[0], float(scale), _stream()))
         return out
     if table.dim() != 2 or table.shape[1] != width or out.dtype != torch.float32:
         raise KernelError(f"embed: table {tuple(table.shape)} / out {tuple(out.shape)} {out.dtype} do not fit")
     lib = core()
     _check(lib, lib.nnis_embed(ids.data_ptr(), table.data_ptr(), _code(table), out.data_ptr(), tokens, width,
-                               table.shape[0], _stream()))
+                               table.shape[0], float(scale), _stream()))
     return out
 
 
@@ -430,10 +453,36 @@ def step_tables(tok_slot: torch.Tensor, tok_pos: torch.Tensor, tokens: int, cos:
     return out
 
 
+class ScoreExtras:
+    """What an attention may do to its scores beyond scale and cap, each off
+    when zero or None.  ``keep_first``: with a window, keys at positions below
+    this stay visible to every later query.  ``bias``: float32 [heads, reach +
+    1], added to the scaled score of a key ``n`` positions back from its
+    query, row min(n, reach) (a table by distance, one column set per head).
+    ``sink``: float32 [heads], a score that joins the softmax's denominator
+    once and has no value (exp(sink) is added to the sum of the weights)."""
+
+    def __init__(self, keep_first: int = 0, bias: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None):
+        self.keep_first, self.bias, self.sink = int(keep_first), bias, sink
+        self.reach = 0 if bias is None else bias.shape[1] - 1
+
+    def __bool__(self) -> bool:
+        return bool(self.keep_first) or self.bias is not None or self.sink is not None
+
+    def check(self, heads: int) -> None:
+        for t, what in ((self.bias, "bias"), (self.sink, "sink")):
+            if t is not None:
+                _dev(t, f"attention {what}")
+                if t.dtype != torch.float32 or t.shape[0] != heads or t.dim() != (2 if what == "bias" else 1):
+                    raise KernelError(f"attention: the {what} must be float32 with a row per head ({heads}), got {tuple(t.shape)} {t.dtype}")
+        if self.keep_first < 0:
+            raise KernelError(f"attention: keep_first must not be negative, got {self.keep_first}")
+
+
 def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                    block_table: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, heads: int, kv_heads: int,
                    head_dim: int, scale: float, window: int = 0, value_dim: Optional[int] = None,
-                   softcap: float = 0.0) -> torch.Tensor:
+                   softcap: float = 0.0, extras: Optional[ScoreExtras] = None) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its slot up to
     its own position (32-bit arithmetic, any storage type).  ``value_dim``:
     channels of a value head and of a head's output (None: as the keys).
@@ -451,6 +500,14 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
     lib = attention_module(head_dim, value_dim, softcap)
+    if extras:
+        extras.check(heads)
+        _check(lib, lib.nnis_attention_rows_more(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
+                                                 v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
+                                                 tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
+                                                 int(window), float(scale), int(value_dim), float(softcap), extras.keep_first,
+                                                 _ptr(extras.bias), extras.reach, _ptr(extras.sink), _stream()))
+        return out
     _check(lib, lib.nnis_attention_rows(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
                                         v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
                                         tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
@@ -1068,7 +1125,7 @@ def prefill_tile_list(new_tokens, first_positions, padded, rows: int):
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
               window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None, plan=None,
-              value_dim: Optional[int] = None, softcap: float = 0.0):
+              value_dim: Optional[int] = None, softcap: float = 0.0, extras: Optional[ScoreExtras] = None):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
     tokens, one for runs of tokens); anything else takes the 32-bit kernel.
@@ -1078,7 +1135,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     (waves, columns) of a step of prompts (``prefill_plan``); None: as those
     functions choose for the step's planned sizes."""
     value_dim = value_dim or head_dim
-    fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap)
+    fast = attention_on_matrix_cores(q.dtype, view.k_pages.dtype, head_dim, value_dim, softcap, extras)
     size = max(head_dim, value_dim)  # what a wave's registers are sized by
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if size <= 64 else (2 if size <= 128 else 1)):
         splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * value_dim)
@@ -1101,12 +1158,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
                                       waves, columns, value_dim, softcap)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
-                          kv_heads, head_dim, scale, window, value_dim, softcap)
+                          kv_heads, head_dim, scale, window, value_dim, softcap, extras)
 
 
-def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0) -> bool:
+def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0,
+                              extras: Optional[ScoreExtras] = None) -> bool:
     """Whether ``attention`` takes the matrix-core kernels for these types and sizes (else the 32-bit row kernel)."""
-    return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
+    return (not extras and q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
             and (value_dim or head_dim) % 16 == 0)
 
 
@@ -1248,7 +1306,7 @@ def branch_mean(branches, weights, biases, eps: float, out: torch.Tensor) -> tor
     return out
 
 
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu": 2}
 
 
 def gated_act(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> torch.Tensor:
@@ -1426,3 +1484,164 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, ep
                                         weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), tokens, heads, dim, float(eps),
                                         _stream()))
     return out
+
+
+# ---------------------------------------------------------------------------
+# the residual's step around a norm without statistics; logits bent by a cap
+# ---------------------------------------------------------------------------
+
+def tanh_norm_step(x: Optional[torch.Tensor], x_out: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None, post=None,
+                   rows_add: Optional[torch.Tensor] = None, vec_add: Optional[torch.Tensor] = None, following=None,
+                   h: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One kernel for what lies between two projections of a layer whose
+    norm is y -> tanh(alpha y) w + b.  ``x``: the 32-bit stream [tokens,
+    width], or None for a stream of zeros (then ``y`` gives the shape).  v = x + (``post`` ? post(y) : y) + rows_add + vec_add, each term
+    only if given; ``x_out`` (x itself, or another tensor of its shape) takes
+    v; ``h`` takes ``following``(v), or v without one.  ``post`` /
+    ``following``: (alpha, weight, bias).  ``rows`` (int32): output row r
+    reads row rows[r]; the stream is then left as it is.  Returns ``h``."""
+    shape_of = x if x is not None else y
+    if shape_of is None or shape_of.dim() != 2:
+        raise KernelError("tanh_norm_step: a stream or an output [tokens, width] is needed")
+    if x is not None:
+        _dev(x, "x")
+        if x.dtype != torch.float32:
+            raise KernelError(f"tanh_norm_step: the stream is float32, got {x.dtype}")
+    tokens, width = shape_of.shape
+    out_rows = tokens
+    if rows is not None:
+        _dev(rows, "rows")
+        if rows.dtype != torch.int32:
+            raise KernelError("tanh_norm_step: rows must be int32")
+        out_rows = rows.numel()
+        if x_out is not None:
+            raise KernelError("tanh_norm_step: a step over a list of rows leaves the stream as it is")
+    for t, what in ((x_out, "x_out"), (rows_add, "rows_add")):
+        if t is not None:
+            _dev(t, what)
+            if t.dtype != torch.float32 or t.shape != shape_of.shape:
+                raise KernelError(f"tanh_norm_step: {what} {tuple(t.shape)} {t.dtype} against the stream {tuple(shape_of.shape)}")
+    if y is not None:
+        _dev(y, "y")
+        if y.shape != shape_of.shape:
+            raise KernelError(f"tanh_norm_step: y {tuple(y.shape)} against the stream {tuple(shape_of.shape)}")
+    w_code = None
+    for norm, what in ((post, "post"), (following, "following")):
+        if norm is not None:
+            _, weight, bias = norm
+            _dev(weight, f"{what} weight"), _dev(bias, f"{what} bias")
+            if weight.numel() != width or bias.numel() != width or weight.dtype != bias.dtype:
+                raise KernelError(f"tanh_norm_step: the {what} norm's weight and bias do not fit a width of {width}")
+            if w_code is not None and _code(weight) != w_code:
+                raise KernelError("tanh_norm_step: the norms' weights differ in type")
+            w_code = _code(weight)
+    if vec_add is not None:
+        _dev(vec_add, "vec_add")
+        if vec_add.numel() != width or (w_code is not None and _code(vec_add) != w_code):
+            raise KernelError(f"tanh_norm_step: the vector does not fit a width of {width} or the weights' type")
+        w_code = _code(vec_add)
+    if post is not None and y is None:
+        raise KernelError("tanh_norm_step: a norm on the way in needs something to norm")
+    if h is not None:
+        _dev(h, "h")
+        if h.shape != (out_rows, width):
+            raise KernelError(f"tanh_norm_step: h {tuple(h.shape)} against {out_rows} rows of {width}")
+    lib = core()
+    _check(lib, lib.nnis_tanh_norm_step(
+        _ptr(x), _ptr(x_out), _ptr(y), _code(y) if y is not None else 0,
+        _ptr(post[1]) if post else None, _ptr(post[2]) if post else None, float(post[0]) if post else 0.0,
+        _ptr(rows_add), _ptr(vec_add), _ptr(following[1]) if following else None, _ptr(following[2]) if following else None,
+        float(following[0]) if following else 0.0, w_code or 0, _ptr(h), _code(h) if h is not None else 0, _ptr(rows),
+        out_rows, width, _stream()))
+    return h
+
+
+def tanh_cap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x -> cap * tanh(x / cap), in place, on 32-bit rows."""
+    _dev(x, "x")
+    if x.dtype != torch.float32 or not cap > 0.0:
+        raise KernelError(f"tanh_cap: 32-bit rows and a positive cap are needed, got {x.dtype} and {cap}")
+    lib = core()
+    _check(lib, lib.nnis_tanh_cap(x.data_ptr(), float(cap), x.numel(), _stream()))
+    return x
+
+
+# ---------------------------------------------------------------------------
+# attention over a cached latent: between the projections
+# ---------------------------------------------------------------------------
+
+def latent_prepare(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, gates: int, q_weight: Optional[torch.Tensor],
+                   c_weight: torch.Tensor, eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                   tok_slot: torch.Tensor, tok_pos: torch.Tensor, cq: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                   v_pages: Optional[torch.Tensor], block_table: Optional[torch.Tensor], gate: Optional[torch.Tensor]) -> None:
+    """From the rows of one fused projection, [query latent (q_rank) | latent
+    (kv_rank) | rotated key part (rot_dim) | gate logits (gates)]: ``cq`` takes
+    the query latent over its root mean square times ``q_weight``; the latent
+    likewise with ``c_weight``, written as the first kv_rank key channels and
+    as the value of each token's place in the pages (one key/value head, keys
+    of kv_rank + rot_dim channels, values of kv_rank), the rotated key part
+    (pairs of neighbouring channels turned by the token's position) behind it
+    in the keys; ``gate`` (float32) takes sigmoid of the gate logits."""
+    _dev(proj, "proj"), _dev(c_weight, "c_weight"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
+    tokens = proj.shape[0]
+    if proj.dim() != 2 or proj.shape[1] != q_rank + kv_rank + rot_dim + gates:
+        raise KernelError(f"latent_prepare: rows of {proj.shape[1]} against {q_rank} + {kv_rank} + {rot_dim} + {gates}")
+    if c_weight.numel() != kv_rank or (q_rank and (q_weight is None or q_weight.numel() != q_rank or q_weight.dtype != c_weight.dtype)):
+        raise KernelError("latent_prepare: the norms' weights do not fit the latents")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or min(tok_slot.numel(), tok_pos.numel()) < tokens:
+        raise KernelError("latent_prepare: tok_slot / tok_pos must be int32 with one entry per token")
+    if q_rank:
+        _dev(cq, "cq")
+        if cq.shape != (tokens, q_rank):
+            raise KernelError(f"latent_prepare: cq {tuple(cq.shape)} against {tokens} rows of {q_rank}")
+    positions = 0
+    if rot_dim:
+        _dev(cos, "cos"), _dev(sin, "sin")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rot_dim // 2:
+            raise KernelError(f"latent_prepare: tables {tuple(cos.shape)} do not fit rot_dim {rot_dim} in float32")
+        positions = cos.shape[0]
+    if gates:
+        _dev(gate, "gate")
+        if gate.dtype != torch.float32 or gate.shape != (tokens, gates):
+            raise KernelError(f"latent_prepare: gate must be float32 [{tokens}, {gates}]")
+    max_pages = cache_code = 0
+    if k_pages is not None:
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
+        if not _pages_fit(k_pages, v_pages, 1, kv_rank + rot_dim, kv_rank) or k_pages.dtype != v_pages.dtype:
+            raise KernelError(f"latent_prepare: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelError("latent_prepare: block_table must be int32 [slots, pages]")
+        max_pages, cache_code = block_table.shape[1], _code(k_pages)
+    lib = latent()
+    _check(lib, lib.nnis_latent_prepare(proj.data_ptr(), _code(proj), tokens, q_rank, kv_rank, rot_dim, gates, _ptr(q_weight),
+                                        c_weight.data_ptr(), _code(c_weight), float(eps), _ptr(cos), _ptr(sin), positions,
+                                        tok_slot.data_ptr(), tok_pos.data_ptr(), _ptr(cq), _code(cq) if cq is not None else 0,
+                                        _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, _ptr(gate), _stream()))
+
+
+def latent_rotate_q(q: torch.Tensor, heads: int, head_width: int, first: int, rot_dim: int, cos: torch.Tensor, sin: torch.Tensor,
+                    tok_pos: torch.Tensor) -> torch.Tensor:
+    """Turns channels [first, first + rot_dim) of every head of ``q`` [tokens,
+    heads * head_width] by each token's position, pairs of neighbouring
+    channels, in place."""
+    _dev(q, "q"), _dev(cos, "cos"), _dev(sin, "sin"), _dev(tok_pos, "tok_pos")
+    tokens = q.shape[0]
+    if q.shape != (tokens, heads * head_width) or tok_pos.dtype != torch.int32 or tok_pos.numel() < tokens:
+        raise KernelError(f"latent_rotate_q: q {tuple(q.shape)} against {heads} heads of {head_width}")
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rot_dim // 2:
+        raise KernelError(f"latent_rotate_q: tables {tuple(cos.shape)} do not fit rot_dim {rot_dim} in float32")
+    lib = latent()
+    _check(lib, lib.nnis_latent_rotate_q(q.data_ptr(), _code(q), tokens, heads, head_width, first, rot_dim, cos.data_ptr(),
+                                         sin.data_ptr(), cos.shape[0], tok_pos.data_ptr(), _stream()))
+    return q
+
+
+def head_scale(o: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
+    """o[t, h, :] *= gate[t, h], in place; ``o`` [tokens, heads * channels], ``gate`` float32 [tokens, heads]."""
+    _dev(o, "o"), _dev(gate, "gate")
+    tokens = o.shape[0]
+    if o.shape[1] % heads or gate.shape != (tokens, heads) or gate.dtype != torch.float32:
+        raise KernelError(f"head_scale: o {tuple(o.shape)} and gate {tuple(gate.shape)} {gate.dtype} do not fit {heads} heads")
+    lib = latent()
+    _check(lib, lib.nnis_head_scale(o.data_ptr(), _code(o), gate.data_ptr(), tokens, heads, o.shape[1] // heads, _stream()))
+    return o

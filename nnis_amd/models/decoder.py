@@ -21,6 +21,9 @@ class DecoderModel:
         self.positions = {name: build_part("position", description) for name, description in spec.positions.items()}
         self.embedding = build_part("embedding", spec.embedding)
         self.layers = [build_part("block", description, positions=self.positions) for description in spec.layers]
+        # what a schedule entry does to the stream before its layer runs, by the entry's index
+        self.entries = {index: build_part("pass_entry", entry.enter) for index, entry in enumerate(spec.schedule)
+                        if entry.enter is not None}
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.bound = False
@@ -29,7 +32,7 @@ class DecoderModel:
 
     # ---- weights -------------------------------------------------------------
     def parts(self):
-        return [self.embedding, *self.positions.values(), *self.layers, self.final_norm, self.head]
+        return [self.embedding, *self.positions.values(), *self.layers, *self.entries.values(), self.final_norm, self.head]
 
     def tensors(self) -> List[TensorSpec]:
         out, seen = [], set()
@@ -56,6 +59,7 @@ class DecoderModel:
         """Bytes of weights a decode step reads: every layer each time the
         schedule runs it, the head, and no embedding table (a row per token)."""
         total = sum(self.layers[entry.layer].weight_bytes() for entry in self.spec.schedule)
+        total += sum(part.weight_bytes() for part in self.entries.values())
         return total + self.final_norm.weight_bytes() + self.head.weight_bytes()
 
     def graph_safe(self) -> bool:
@@ -119,13 +123,25 @@ class DecoderModel:
             x = self.embedding.forward(ids, ctx.tokens, rt)
         for position in self.positions.values():
             x = position.embed(x, ctx, rt)
+        from ..parts.lazy import PostNormed
+
+        embedded = None
+        if any(part.needs_embedding for part in self.entries.values()):
+            # kept as it is for the entries that add it again: an entry writes a stream that still is this tensor into
+            # a new one; a layer that runs first would write into it
+            embedded = x if 0 in self.entries else x.clone()
         stream = (x, None)
         schedule = self.spec.schedule
         for index, entry in enumerate(schedule):
             layer = self.layers[entry.layer]
+            if index in self.entries:
+                stream = self.entries[index].forward(stream, embedded, rt, following=getattr(layer, "entry_norm", None))
+            elif (isinstance(stream, tuple) and isinstance(stream[1], PostNormed) and not getattr(layer, "takes_post_normed", False)):
+                stream = (stream[0], stream[1].materialize(rt))  # (a block that knows nothing of norms still owed)
             # a block may prepare the first norm of the block that comes next, if that block shows it one
+            # (not across a pass's entry, which changes the stream in between and runs that norm itself)
             following = None
-            if index + 1 < len(schedule) and getattr(layer, "entry_norm", None) is not None:
+            if index + 1 < len(schedule) and index + 1 not in self.entries and getattr(layer, "entry_norm", None) is not None:
                 following = getattr(self.layers[schedule[index + 1].layer], "entry_norm", None)
             if following is not None:
                 stream = layer.forward(stream, ctx, cache.view(index), rt, following=following)
@@ -134,6 +150,8 @@ class DecoderModel:
         x, pending = stream
         if want_rows.shape[0] == 0:
             return rt.empty(0, self.spec.vocab_size, dtype=torch.float32)
+        if isinstance(pending, PostNormed) and not hasattr(self.final_norm, "triple"):
+            pending = pending.materialize(rt)
         if pending is None:
             normed = self.final_norm.forward(x, rt, rows=want_rows)
         else:

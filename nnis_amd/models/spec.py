@@ -19,10 +19,13 @@ class ScheduleEntry:
     """One run of a layer.  ``layer`` indexes ``ModelSpec.layers`` and may
     appear in several entries (shared weights).  ``reads_cache_of`` is the
     index of an earlier schedule entry whose cache this run reads instead of
-    keeping one of its own (it then writes nothing)."""
+    keeping one of its own (it then writes nothing).  ``enter`` describes
+    what is done to the residual stream before the layer runs (a part of role
+    ``pass_entry``: the start of a pass through layers that run several times)."""
 
     layer: int
     reads_cache_of: Optional[int] = None
+    enter: Optional[Dict[str, Any]] = None
 
 
 @dataclass

@@ -8,6 +8,7 @@ from .base import (  # noqa: F401
     Mixer,
     Norm,
     Part,
+    PassEntry,
     PositionEncoding,
     RotaryTables,
     StateRequest,
@@ -16,4 +17,4 @@ from .base import (  # noqa: F401
     register_part,
     registered_kinds,
 )
-from . import attention, block, embedding, feedforward, norm, recurrent, rope  # noqa: F401
+from . import attention, block, embedding, entry, feedforward, latent, norm, recurrent, rope  # noqa: F401

@@ -10,7 +10,10 @@ on the four projections; values (and a head's output) of another size than
 the keys (``value_dim``); a scale of the scores other than 1 / sqrt(head_dim);
 scores bent by a cap, s -> softcap * tanh(s / softcap), before the softmax;
 a rotation of the first channels of a head only (the position encoding's
-``rot_dim``).
+``rot_dim``); with a window, first tokens that stay visible to every later
+query (``keep_first``); a learned bias by distance added to the scaled score
+(``distance_bias``, ``bias_reach``); a sink in the softmax's denominator
+(``sink``).
 """
 
 from __future__ import annotations
@@ -24,11 +27,30 @@ from .base import KVRequest, Mixer, TensorSpec, register_part
 from .linear import Projection
 
 
+def distance_bucket(n: int, buckets: int, reach: int) -> int:
+    """The row of a table of ``buckets`` rows that a key ``n`` positions back
+    reads: the distance itself in the first half of the table, then steps that
+    widen with the logarithm of the distance, so that the last row is met at
+    ``reach`` and holds for everything beyond."""
+    half = buckets // 2
+    if n < half:
+        return n
+    return min(buckets - 1, half + int(math.floor(math.log(n / half) / math.log(reach / half) * (buckets - half))))
+
+
 class CausalSelfAttention(Mixer):
     graph_safe = True
 
     def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None,
-                 value_dim=None, scale=None, softcap=None, q_bias=None, k_bias=None, v_bias=None, o_bias=None):
+                 value_dim=None, scale=None, softcap=None, q_bias=None, k_bias=None, v_bias=None, o_bias=None,
+                 keep_first=None, distance_bias=None, bias_reach=None, bias_buckets=None, sink=None):
+        """``keep_first``: with a ``window``, keys at positions below it stay
+        visible.  ``distance_bias``: the name of a table [buckets, heads]; the
+        scaled score of a key n positions back gets row ``distance_bucket(n,
+        buckets, bias_reach)`` of its head's column added (the table's length
+        is the checkpoint's; a random model names it as ``bias_buckets``).
+        ``sink``: "zero" for a score of 0, or the name of a tensor [heads] of
+        learned scores, that joins the softmax's denominator and has no value."""
         if heads % kv_heads != 0:
             raise InvalidInput(f"{heads} query heads do not divide into {kv_heads} key/value heads")
         self.width, self.heads, self.kv_heads, self.head_dim = int(width), int(heads), int(kv_heads), int(head_dim)
@@ -53,6 +75,15 @@ class CausalSelfAttention(Mixer):
         self.scale = 1.0 / math.sqrt(self.head_dim) if scale is None else float(scale)  # runtime.rs:943
         if not self.scale > 0.0:
             raise InvalidInput(f"the scale of the scores must be positive, got {scale}")
+        self.keep_first = 0 if not keep_first else int(keep_first)
+        if self.keep_first < 0 or (self.keep_first and not self.window):
+            raise InvalidInput(f"first tokens are kept visible ({keep_first}) beside a window only")
+        self.bias_name, self.bias_reach = distance_bias, None if bias_reach is None else int(bias_reach)
+        self.bias_buckets = None if bias_buckets is None else int(bias_buckets)
+        if distance_bias is not None and (self.bias_reach is None or self.bias_reach < 1):
+            raise InvalidInput(f"a bias by distance needs the distance at which its last row is met, got {bias_reach!r}")
+        self.sink_name = sink
+        self.extras = None  # ``ops.ScoreExtras``, made when the weights are bound
         self.qkv = None
         self.out = None
 
@@ -68,6 +99,10 @@ class CausalSelfAttention(Mixer):
         for key, size in (("q", q_width), ("k", kv_width), ("v", v_width), ("o", self.width)):
             if self.bias_names[key]:
                 out.append(TensorSpec(self.bias_names[key], (size,)))
+        if self.bias_name:
+            out.append(TensorSpec(self.bias_name, (self.bias_buckets, self.heads)))
+        if self.sink_name and self.sink_name != "zero":
+            out.append(TensorSpec(self.sink_name, (self.heads,)))
         return out
 
     def bind(self, weights, rt):
@@ -78,6 +113,20 @@ class CausalSelfAttention(Mixer):
             self.qkv_bias = torch.cat([weights[self.bias_names[key]] for key in ("q", "k", "v")]).contiguous()
         if self.bias_names["o"]:
             self.output_bias = weights[self.bias_names["o"]].contiguous()
+        bias = sink = None
+        if self.bias_name:
+            # the table by bucket becomes a table by distance, [heads, reach + 1] in 32-bit: the kernels index it by min(n, reach)
+            table = weights[self.bias_name].float()
+            buckets = table.shape[0]
+            if buckets < 2 or self.bias_reach <= buckets // 2:
+                raise InvalidInput(f"a bias table of {buckets} rows cannot reach a distance of {self.bias_reach}")
+            rows = torch.tensor([distance_bucket(n, buckets, self.bias_reach) for n in range(self.bias_reach + 1)],
+                                dtype=torch.long, device=table.device)
+            bias = table[rows].t().contiguous()
+        if self.sink_name:
+            sink = (torch.zeros(self.heads, dtype=torch.float32, device=rt.device) if self.sink_name == "zero"
+                    else weights[self.sink_name].float().contiguous())
+        self.extras = rt.ops.ScoreExtras(self.keep_first, bias, sink)
 
     def weight_bytes(self):
         return self.qkv.weight_bytes() + self.out.weight_bytes()
@@ -93,7 +142,7 @@ class CausalSelfAttention(Mixer):
             raise InvalidInput(f"a rotation of {rot_dim} channels does not fit heads of {self.head_dim}")
 
     def _matrix_cores(self, rt) -> bool:
-        return rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap)
+        return rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_dim, self.value_dim, self.softcap, self.extras)
 
     @property
     def _plain(self) -> bool:
@@ -167,7 +216,7 @@ class CausalSelfAttention(Mixer):
                     else self.prompt_plan(ctx.batch, ctx.planned_rows, ctx.planned_len, rt))
         attn = rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0,
                                 keep_runs=into is not None and self.output_bias is None, tables=step, plan=plan,
-                                value_dim=self.value_dim, softcap=self.softcap)
+                                value_dim=self.value_dim, softcap=self.softcap, extras=self.extras)
         if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
             attn = attn.combine()
         if into is not None and self.output_bias is None and into.can_take(attn, self.out.weight):

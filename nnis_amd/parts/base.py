@@ -35,6 +35,11 @@ The interfaces:
 ``Block``
     ``forward(stream, ctx, view, rt)`` -> stream; the block owns the
     arrangement of norm, mixer and feed-forward around the residual stream.
+``PassEntry``
+    ``forward(stream, embedded, rt, following=None)`` -> stream: what a
+    schedule entry does to the stream before its layer runs (the start of a
+    pass through layers that run several times); ``embedded`` is the
+    embedding's output, kept for entries that ask for it (``needs_embedding``).
 """
 
 from __future__ import annotations
@@ -210,12 +215,19 @@ class Block(Part):
         raise NotImplementedError
 
 
+class PassEntry(Part):
+    needs_embedding = False
+
+    def forward(self, stream, embedded, rt, following=None):
+        raise NotImplementedError
+
+
 # --------------------------------------------------------------------------
 # registry of part kinds
 # --------------------------------------------------------------------------
 
 _PART_KINDS: Dict[Tuple[str, str], Callable[..., Part]] = {}
-_ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+_ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head", "pass_entry")
 
 
 def register_part(role: str, kind: str, factory: Callable[..., Part], replace: bool = False) -> None:

@@ -20,7 +20,7 @@ import torch
 from ..errors import InvalidInput
 from ..weights.random_init import register_init_rule
 from .base import Block, TensorSpec, build_part, register_part
-from .lazy import PendingNorm, PreparedStreams, ResidualInto
+from .lazy import PendingNorm, PostNormed, PreparedRows, PreparedStreams, ResidualInto
 
 
 def _joined(plans):
@@ -196,6 +196,96 @@ class HyperConnectionBlock(Block):
         return x, None
 
 
+class PrePostNormBlock(Block):
+    """A layer that norms each sublayer on the way in and on the way out:
+
+        x <- x + post1(mixer(norm1(x)));   x <- x + post2(feed_forward(norm2(x)))
+
+    (the second line only with a feed-forward).  With norms that need no
+    statistics (``TanhNorm``) everything between two sublayers -- the norm on
+    the way out, the sum into the 32-bit stream, the next norm on the way in --
+    is one kernel, and the layer's last output is handed on not yet normed
+    (``PostNormed``), so that whoever takes the stream next does the same in
+    its own first kernel; with other norms each step is the norm's own."""
+
+    takes_post_normed = True
+
+    def __init__(self, width, norm1, post1, mixer, norm2=None, post2=None, feed_forward=None, positions=None):
+        self.width = int(width)
+        if (feed_forward is None) != (norm2 is None) or (feed_forward is None) != (post2 is None):
+            raise InvalidInput("a feed-forward comes with its two norms, or none of the three")
+        self.norm1 = build_part("norm", norm1)
+        self.post1 = build_part("norm", post1)
+        self.mixer = build_part("mixer", mixer, positions=positions)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.post2 = build_part("norm", post2) if post2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        self._parts = [part for part in (self.norm1, self.post1, self.mixer, self.norm2, self.post2, self.feed_forward) if part is not None]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self._parts)
+
+    def tensors(self):
+        return [spec for part in self._parts for spec in part.tensors()]
+
+    def bind(self, weights, rt):
+        for part in self._parts:
+            part.bind(weights, rt)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for part in self._parts)
+
+    def cache_request(self):
+        return self.mixer.cache_request()
+
+    def check(self, rt):
+        for part in self._parts:
+            part.check(rt)
+
+    def decode_plan(self, batch, longest, rt):
+        return _joined(part.decode_plan(batch, longest, rt) for part in self._parts)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        return _joined(part.prompt_plan(batch, rows, longest, rt) for part in self._parts)
+
+    def held_buffers(self, rt):
+        return [buffer for part in self._parts for buffer in part.held_buffers(rt)]
+
+    @property
+    def entry_norm(self):
+        return self.norm1
+
+    @staticmethod
+    def _between(x, y, post, following, rt):
+        """x += post(y) in place; returns following(x)."""
+        if hasattr(post, "triple") and hasattr(following, "triple"):
+            return rt.ops.tanh_norm_step(x, x_out=x, y=y, post=post.triple(), following=following.triple(),
+                                         h=rt.empty(x.shape[0], x.shape[1]))
+        return following.add_forward(x, post.forward(y, rt), rt)
+
+    def forward(self, stream, ctx, view, rt, following=None):
+        """stream: (x, pending) -- pending a tensor, a ``PostNormed`` or None -- or
+        this block's first norm already run (``PreparedRows``).  following: the next
+        block's first norm; run here and handed on if it is of the kind that this
+        block's kernel takes, else the stream goes on as (x, ``PostNormed``)."""
+        if isinstance(stream, PreparedRows):
+            if stream.norm is not self.norm1:
+                raise ValueError("the rows handed to a block are not those of the block's own first norm")
+            x, h = stream.x, stream.h
+        else:
+            x, pending = stream
+            if isinstance(pending, PostNormed) and not hasattr(self.norm1, "triple"):
+                pending = pending.materialize(rt)
+            h = self.norm1.forward(x, rt) if pending is None else self.norm1.add_forward(x, pending, rt)
+        y = self.mixer.forward(h, ctx, view, rt)
+        post = self.post1
+        if self.feed_forward is not None:
+            h = self._between(x, y, self.post1, self.norm2, rt)
+            y = self.feed_forward.forward(h, ctx, rt)
+            post = self.post2
+        if following is not None and hasattr(post, "triple") and hasattr(following, "triple"):
+            return PreparedRows(following, x, self._between(x, y, post, following, rt))
+        return x, PostNormed(y, post)
+
+
 def _noise(spec, generator):
     return torch.randn(tuple(spec.shape), generator=generator, dtype=torch.float32)
 
@@ -206,3 +296,4 @@ register_init_rule("stream_share", lambda spec, generator, dtype: (0.5 + 0.25 * 
 
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "hyper_connections", HyperConnectionBlock)
+register_part("block", "pre_post_norm", PrePostNormBlock)

@@ -15,8 +15,9 @@ from .linear import Projection
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size, width, weight):
-        self.vocab_size, self.width, self.weight_name = int(vocab_size), int(width), weight
+    def __init__(self, vocab_size, width, weight, scale=1.0):
+        """``scale``: every row is multiplied by it on the way out (in 32-bit)."""
+        self.vocab_size, self.width, self.weight_name, self.scale = int(vocab_size), int(width), weight, float(scale)
         self.table = None
 
     def tensors(self):
@@ -37,7 +38,7 @@ class TokenEmbedding(Part):
 
     def forward(self, ids, tokens, rt):
         """ids: int32 on the device -> the 32-bit residual stream [tokens, width]."""
-        return rt.ops.embed(ids, self.table, rt.empty(tokens, self.width, dtype=torch.float32))
+        return rt.ops.embed(ids, self.table, rt.empty(tokens, self.width, dtype=torch.float32), self.scale)
 
 
 class PairHashEmbedding(Part):
@@ -76,8 +77,10 @@ class PairHashEmbedding(Part):
 class LinearHead(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size, width, weight, tied_to=None):
+    def __init__(self, vocab_size, width, weight, tied_to=None, softcap=None):
+        """``softcap``: logits z leave as softcap * tanh(z / softcap)."""
         self.vocab_size, self.width, self.weight_name, self.tied_to = int(vocab_size), int(width), weight, tied_to
+        self.softcap = None if not softcap else float(softcap)
         self.projection = None
 
     def tensors(self):
@@ -95,7 +98,8 @@ class LinearHead(Part):
 
     def forward(self, x, rt):
         """Logits are 32-bit whatever the storage type."""
-        return self.projection(x, rt, out_dtype=torch.float32)
+        logits = self.projection(x, rt, out_dtype=torch.float32)
+        return logits if self.softcap is None else rt.ops.tanh_cap(logits, self.softcap)
 
 
 register_part("embedding", "table", TokenEmbedding)

@@ -1,7 +1,7 @@
 """Gated feed-forward: down( act(gate x) * up x ), act = SiLU
 (/root/reference/crates/nnis-model/src/runtime.rs:1054-1087;
-/root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28) or the tanh form
-of GELU.  Gate and up are one fused projection whose first ``inner`` output
+/root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28), the tanh form
+of GELU, or ReLU.  Gate and up are one fused projection whose first ``inner`` output
 columns are the gate."""
 
 from __future__ import annotations
@@ -17,8 +17,8 @@ class GatedFeedForward(FeedForward):
     graph_safe = True
 
     def __init__(self, width, inner, gate, up, down, activation="silu"):
-        if activation not in ("silu", "gelu_tanh"):
-            raise Unsupported(f"gated feed-forward activation {activation!r}; silu and gelu_tanh are built")
+        if activation not in ("silu", "gelu_tanh", "relu"):
+            raise Unsupported(f"gated feed-forward activation {activation!r}; silu, gelu_tanh and relu are built")
         self.activation = activation
         self.width, self.inner = int(width), int(inner)
         self.names = {"gate": gate, "up": up, "down": down}

@@ -116,3 +116,27 @@ class PreparedStreams:
 
     def __init__(self, norm, x: torch.Tensor, h: torch.Tensor):
         self.norm, self.x, self.h = norm, x, h
+
+
+class PostNormed:
+    """A part's output ``y`` whose norm has not run: what is to be added to
+    the residual stream is ``norm(y)``.  A layer that norms its sublayers on
+    the way out too hands this on as the stream's pending part, so that
+    whoever takes the stream next (a block, a pass's entry, the final norm)
+    does norm, sum and its own first step in one kernel; anybody else calls
+    ``materialize``."""
+
+    def __init__(self, y: torch.Tensor, norm):
+        self.y, self.norm = y, norm
+
+    def materialize(self, rt) -> torch.Tensor:
+        return self.norm.forward(self.y, rt)
+
+
+class PreparedRows:
+    """A stream ``x`` [tokens, width] with nothing left to add, and ``h``,
+    the rows that ``norm`` -- the first norm of the block that takes this --
+    makes of it: run already by whoever wrote the stream last."""
+
+    def __init__(self, norm, x: torch.Tensor, h: torch.Tensor):
+        self.norm, self.x, self.h = norm, x, h

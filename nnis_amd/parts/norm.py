@@ -3,6 +3,9 @@
 
 from __future__ import annotations
 
+import torch
+
+from ..weights.random_init import register_init_rule
 from .base import Norm, TensorSpec, register_part
 
 
@@ -97,3 +100,62 @@ class LayerNorm(Norm):
 
 
 register_part("norm", "layer", LayerNorm)
+
+
+class TanhNorm(Norm):
+    """A norm without statistics: y = tanh(alpha x) * w + b, ``alpha`` one
+    learned number, ``w`` and ``b`` per channel.  Nothing of a row is summed,
+    so it rides in any kernel that touches the row once: ``ops.tanh_norm_step``
+    takes a sublayer's output through one such norm into the stream and the
+    stream through another into the next sublayer's input.  ``triple()`` is
+    what that kernel needs of a norm."""
+
+    graph_safe = True
+
+    def __init__(self, width: int, weight: str, bias: str, alpha: str):
+        self.width = int(width)
+        self.weight_name, self.bias_name, self.alpha_name = weight, bias, alpha
+        self.weight = self.bias = None
+        self.alpha = 1.0
+
+    def tensors(self):
+        return [TensorSpec(self.weight_name, (self.width,), init="gain"), TensorSpec(self.bias_name, (self.width,)),
+                TensorSpec(self.alpha_name, (), init="tanh_alpha")]
+
+    def bind(self, weights, rt):
+        self.weight = weights[self.weight_name].contiguous()
+        self.bias = weights[self.bias_name].to(self.weight.dtype).contiguous()
+        self.alpha = float(weights[self.alpha_name].float().item())  # (a kernel argument: read once, when the model is loaded)
+
+    def weight_bytes(self):
+        return 2 * self.weight.numel() * self.weight.element_size()
+
+    def triple(self):
+        return self.alpha, self.weight, self.bias
+
+    def forward(self, x, rt, rows=None):
+        count = x.shape[0] if rows is None else rows.shape[0]
+        out = rt.empty(count, self.width)
+        if x.dtype == torch.float32:
+            return rt.ops.tanh_norm_step(x, following=self.triple(), h=out, rows=rows)
+        return rt.ops.tanh_norm_step(None, y=x, following=self.triple(), h=out, rows=rows)  # rows in the activation type
+
+    def add_forward(self, residual, delta, rt, rows=None):
+        """``delta``: a tensor, or a ``PostNormed`` (its norm then runs in the same kernel if it is of this kind)."""
+        from .lazy import PostNormed
+
+        post = None
+        if isinstance(delta, PostNormed):
+            if hasattr(delta.norm, "triple"):
+                delta, post = delta.y, delta.norm.triple()
+            else:
+                delta = delta.materialize(rt)
+        count = residual.shape[0] if rows is None else rows.shape[0]
+        return rt.ops.tanh_norm_step(residual, x_out=residual if rows is None else None, y=delta, post=post,
+                                     following=self.triple(), h=rt.empty(count, self.width), rows=rows)
+
+
+# what a random model draws for alpha: around one half, so that tanh bends the stream's larger entries
+register_init_rule("tanh_alpha", lambda spec, generator, dtype: (0.5 + 0.05 * torch.randn(tuple(spec.shape), generator=generator)).to(dtype),
+                   replace=True)
+register_part("norm", "dynamic_tanh", TanhNorm)

@@ -37,6 +37,7 @@ def rotary_tables(positions: int, rot_dim: int, theta: float, angles: str = "flo
 
 class RotaryHalf(PositionEncoding):
     graph_safe = True
+    pairing = "halves"  # channel i turns with channel i + rot_dim / 2
 
     def __init__(self, rot_dim: int, theta: float, max_positions: int = None, angles: str = "float32"):
         """``max_positions`` None: the model names no last position; the tables
@@ -73,3 +74,14 @@ class RotaryHalf(PositionEncoding):
 
 
 register_part("position", "rotary_half", RotaryHalf)
+
+
+class RotaryPairs(RotaryHalf):
+    """The same tables (angle = position x frequency i) for consumers that
+    turn channel 2i with channel 2i + 1.  Which channels make a pair is the
+    consuming kernel's business: it asks for the ``pairing`` it implements."""
+
+    pairing = "neighbours"
+
+
+register_part("position", "rotary_pairs", RotaryPairs)

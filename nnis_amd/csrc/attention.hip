@@ -49,6 +49,12 @@ constexpr int HDR = NNIS_REG_DIM;
 #ifndef NNIS_SCORE_CAP
 #define NNIS_SCORE_CAP 0
 #endif
+// 1: the matrix-core kernels also take what AttnArgs lists beyond the plain formula (first keys kept visible beside a
+// window, a bias by distance, a sink in the denominator); compiled in, like the cap, so that the kernels of plain
+// scores stay the code they are
+#ifndef NNIS_SCORE_EXTRAS
+#define NNIS_SCORE_EXTRAS 0
+#endif
 
 struct AttnArgs {
   const void* q;  // [tokens, heads, HD]
@@ -348,6 +354,78 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
   }
 }
 
+// What a wave needs beyond lo and hi where the module takes the extras: the row of the bias table of each
+// column's head (null without a bias; a column's query sits at hi[c], so a key's distance is hi[c] - key), how
+// far the table reaches, and how many first keys stay visible below a window's lower end.
+template <int C>
+struct More {
+#if NNIS_SCORE_EXTRAS
+  const float* bias_row[C];
+  int reach;
+  int keep;
+#endif
+};
+
+#if NNIS_SCORE_EXTRAS
+// attend_block with the extras: a key counts if it is at or below the column's position and inside the window or
+// among the kept first keys; the bias by distance joins the scaled score (both in base-2 units) before the maximum.
+template <int C>
+__device__ __forceinline__ void attend_block_more(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, int key0,
+                                                  const int (&lo)[C], const int (&hi)[C], float scale_log2, const ScoreCap& cap,
+                                                  const More<C>& more, int g) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    f32x4 s[2];
+    float block_max = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[t] = score_tile(f.keys[t], q[c]);
+      bend(s[t], cap);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + 8 * g + 4 * t + e;
+        const bool seen = key <= hi[c] && (key >= lo[c] || key < more.keep);
+        float v = s[t][e] * scale_log2;
+        if (more.bias_row[c] != nullptr && seen) v = fmaf(more.bias_row[c][min(hi[c] - key, more.reach)], kLog2e, v);
+        s[t][e] = seen ? v : -INFINITY;
+        block_max = fmaxf(block_max, s[t][e]);
+      }
+    }
+    if (__any(block_max > st.m[c] + kLazyRise)) {  // (see attend_block)
+      float moved = fmaxf(st.m[c], block_max);
+      moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
+      moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
+      const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
+      st.l[c] *= shrink;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
+      st.m[c] = moved;
+    }
+    const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];
+    bf16x8 p;
+    float sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = __builtin_amdgcn_exp2f(s[t][e] - base);  // -inf for a key that does not count: 0
+        sum += w;
+        p[4 * t + e] = (__bf16)w;
+      }
+    st.l[c] += sum;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t)
+      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
+  }
+}
+
+// The sink joins a column's sum once, where the sum is final (or in the first run of a key range that is cut
+// into runs): 2^(sink log2 e - reference), the reference being what the sum's terms are taken against.
+__device__ __forceinline__ float sink_term(const float* sink, int head, float reference) {
+  return sink == nullptr ? 0.0f : __builtin_amdgcn_exp2f(sink[head] * kLog2e - reference);
+}
+#endif
+
 // The same work with the matrix unit and the vector unit side by side, for blocks all of whose keys count for
 // every column (no key is looked at).  A unit is one block's 32 keys for one column tile: 2 * (HD / 32) matrix
 // instructions for its scores, then the softmax's vector work on them (eight exponentials of 16 cycles a wave
@@ -490,6 +568,11 @@ struct MfmaArgs {
   const int* tok_pos;     // [tokens]
   int splits, heads_first;
   float* partial;         // [tokens, heads, splits, kPartial] when splits > 1: HD outputs, maximum, sum
+  // with NNIS_SCORE_EXTRAS (see AttnArgs): each off when zero or null
+  int keep_first;
+  const float* bias;      // [heads, reach + 1], in the scores' own units (natural logarithm)
+  int reach;
+  const float* sink;      // [heads]
 };
 
 __device__ __forceinline__ const bf16_t* k_page_ptr(const MfmaArgs& a, int page, int kv_head) {
@@ -586,7 +669,7 @@ __device__ __forceinline__ bool merge_group(AttnState<C>& st, float* slots, int 
 template <int C, int RING>
 __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
                                            int kv_head, int first, int stride, int mine, int last_key,
-                                           const int (&lo)[C], const int (&hi)[C], int lane) {
+                                           const int (&lo)[C], const int (&hi)[C], int lane, const More<C>& more) {
   // (The run's bounds are the same in every lane -- they come from sums over the wave -- but the compiler has them
   // in vector registers unless it is told: as scalars the loop's counters, the pages' numbers and the pages'
   // addresses cost no vector instruction, of which the loop has none to spare.)
@@ -616,7 +699,11 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
     load_block(into, k_base + page * k_page_stride, v_base + page * v_page_stride, b & 1, r, g);
   };
   auto work = [&](const BlockFrags& f, int b) {
+#if NNIS_SCORE_EXTRAS
+    attend_block_more<C>(st, q, f, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, a.cap, more, g);
+#else
     attend_block<C>(st, q, f, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, a.cap, g);
+#endif
   };
   int b0 = 0;
   if (blocks >= 2 * RING) {
@@ -644,7 +731,11 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   every_lo = __builtin_amdgcn_readfirstlane(every_lo);
   every_hi = __builtin_amdgcn_readfirstlane(every_hi);
   const int whole_pages = (every_hi + 1) / kPageTokens;  // pages 0 .. whole_pages - 1 of the sequence end at or below every_hi
+#if NNIS_SCORE_EXTRAS
+  const int inner_end = 0;  // (every block goes through the loop that looks at its keys: their distances decide their bias)
+#else
   const int inner_end = whole_pages > first ? 2 * min(mine, (whole_pages - first + stride - 1) / stride) : 0;  // in blocks of the run
+#endif
   const int low_page = (every_lo + kPageTokens - 1) / kPageTokens;
   int inner_begin = low_page > first ? 2 * ((low_page - first + stride - 1) / stride) : 0;
   inner_begin = (inner_begin + RING - 1) / RING * RING;  // whole rounds of the ring
@@ -774,10 +865,28 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     }
     AttnState<C> st;
     init_state(st);
+    More<C> more;
+#if NNIS_SCORE_EXTRAS
+    more.reach = a.reach;
+    more.keep = a.window > 0 ? a.keep_first : 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int head = min(head0 + c % GH, a.heads - 1);
+      more.bias_row[c] = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
+    }
+#endif
     if (last >= 0) {
       const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
+#if NNIS_SCORE_EXTRAS
+      // the pages of the kept first keys that lie before the window's first page, dealt like the window's
+      const int kept_pages = min(first_page, (more.keep + kPageTokens - 1) / kPageTokens);
+      if (kept_pages > 0) {
+        const int mine_kept = kept_pages > index ? (kept_pages - index + size - 1) / size : 0;
+        attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, index, size, mine_kept, more.keep - 1, lo, hi, lane, more);
+      }
+#endif
       const int mine = page_count > index ? (page_count - index + size - 1) / size : 0;  // pages of this wave
-      attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + index, size, mine, last, lo, hi, lane);
+      attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + index, size, mine, last, lo, hi, lane, more);
     }
     if (!merge_group<C>(st, slots, index, size, rounds, lane)) return;
 #pragma unroll
@@ -789,6 +898,9 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
         total += __shfl_xor(total, 16, kWave);
         total += __shfl_xor(total, 32, kWave);
         if (!live[c]) continue;
+#if NNIS_SCORE_EXTRAS
+        total += sink_term(a.sink, head0 + gh, st.m[c]);
+#endif
         const float inv = 1.0f / total;
         bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HDV;
 #pragma unroll
@@ -847,6 +959,10 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
     total[c] = st.l[c];
     total[c] += __shfl_xor(total[c], 16, kWave);
     total[c] += __shfl_xor(total[c], 32, kWave);
+#if NNIS_SCORE_EXTRAS
+    // (the first run of a token's keys always holds its first page, so its reference is a score's own size)
+    if (live[c] && split == 0) total[c] += sink_term(a.sink, kv_head * group + 16 * c + r, st.m[c]);
+#endif
   }
   if (a.splits == 1) {
 #pragma unroll
@@ -917,8 +1033,24 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(Mfma
   const int end = min(begin + per_split, page_first + page_count);
   AttnState<C> st;
   init_state(st);
+  More<C> more;
+#if NNIS_SCORE_EXTRAS
+  more.reach = a.reach;
+  more.keep = a.window > 0 ? a.keep_first : 0;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int head = kv_head * group + (live[c] ? 16 * c + r : 0);
+    more.bias_row[c] = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
+  }
+  // the pages of the kept first keys that lie before the window's first page go with the first run of the keys
+  const int kept_pages = split == 0 ? min(page_first, (more.keep + kPageTokens - 1) / kPageTokens) : 0;
+  if (kept_pages > 0) {
+    const int mine_kept = kept_pages > wave ? (kept_pages - wave + waves - 1) / waves : 0;
+    attend_run<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pages, kv_head, wave, waves, mine_kept, more.keep - 1, lo, hi, lane, more);
+  }
+#endif
   const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // pages of this wave
-  attend_run<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane);
+  attend_run<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane, more);
   finish_decode<C>(st, live, a, merge, token, kv_head, split, wave, waves, lane);
 }
 
@@ -1234,6 +1366,15 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
   a.cap.out = softcap * kLog2e;
   a.tile_seq = a.tile_row0 = a.seq_slot = a.seq_start = a.seq_pos0 = a.tok_slot = a.tok_pos = nullptr;
   a.splits = 1; a.heads_first = 0; a.partial = nullptr; a.rows_by_token = 0;
+  a.keep_first = 0; a.bias = nullptr; a.reach = 0; a.sink = nullptr;
+  return 0;
+}
+
+int fill_extras(MfmaArgs& a, int keep_first, const float* bias, int reach, const float* sink) {
+  NNIS_REQUIRE(NNIS_SCORE_EXTRAS || (keep_first == 0 && bias == nullptr && sink == nullptr),
+               "attention: this module is compiled without kept first keys, a bias by distance and a sink");
+  NNIS_REQUIRE(keep_first >= 0 && (bias == nullptr || reach >= 0), "attention: bad keep_first %d or reach %d", keep_first, reach);
+  a.keep_first = a.window > 0 ? keep_first : 0; a.bias = bias; a.reach = reach; a.sink = sink;
   return 0;
 }
 }  // namespace
@@ -1282,13 +1423,15 @@ extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int col
   return waves;
 }
 
-extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
-                                           const int* block_table, int max_pages, const int* tile_seq,
-                                           const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
-                                           const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
-                                           float scale, int waves, int columns, float softcap, void* stream) {
+extern "C" int nnis_attention_prefill_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                                const int* block_table, int max_pages, const int* tile_seq,
+                                                const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
+                                                const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
+                                                float scale, int waves, int columns, float softcap, int keep_first,
+                                                const float* bias, int reach, const float* sink, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
+  if (fill_extras(a, keep_first, bias, reach, sink)) return 1;
   if (tiles <= 0) return 0;
   a.tile_seq = tile_seq; a.tile_row0 = tile_row0; a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0;
   const int group = heads / kv_heads;
@@ -1363,13 +1506,15 @@ extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
 // for columns or keys on lanes and fail where that kernel does not take the sizes.  combine: 0 leaves the
 // runs in `partial` ([tokens, heads, splits, head_dim + 4]: outputs, reference, sum) and writes no output: the
 // projection that follows, or nnis_attention_combine, adds them up.
-extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
-                                          const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
-                                          int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                          int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
-                                          float softcap, void* stream) {
+extern "C" int nnis_attention_decode_bf16_more(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                               const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
+                                               int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
+                                               int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
+                                               float softcap, int keep_first, const float* bias, int reach, const float* sink,
+                                               void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale, softcap)) return 1;
+  if (fill_extras(a, keep_first, bias, reach, sink)) return 1;
   a.rows_by_token = rows_by_token ? 1 : 0;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
@@ -1383,7 +1528,7 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   NNIS_REQUIRE(group <= 16 * kMaxColumns, "attention: a group of %d query heads is more than this head size's decode kernel carries (%d)",
                group, 16 * kMaxColumns);
   NNIS_REQUIRE(kind >= 0 && kind <= 2, "attention: unknown decode kernel %d", kind);
-  const bool keys_fit = group <= 4 && HDR <= kKeysMaxHD;
+  const bool keys_fit = !NNIS_SCORE_EXTRAS && group <= 4 && HDR <= kKeysMaxHD;  // (the kernel with keys on lanes knows no extras)
   NNIS_REQUIRE(kind != 2 || keys_fit, "attention: the kernel with keys on lanes takes groups of up to 4 heads of up to %d channels",
                kKeysMaxHD);
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.splits = splits; a.partial = partial;
@@ -1425,6 +1570,26 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   return 0;
 }
 
+extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                          const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
+                                          int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
+                                          int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
+                                          float softcap, void* stream) {
+  return nnis_attention_decode_bf16_more(q, out, k_pages, v_pages, block_table, max_pages, tok_slot, tok_pos, tokens, heads, kv_heads,
+                                         head_dim, window, scale, splits, waves, partial, kind, combine, rows_by_token, softcap, 0,
+                                         nullptr, 0, nullptr, stream);
+}
+
+extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                           const int* block_table, int max_pages, const int* tile_seq,
+                                           const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
+                                           const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
+                                           float scale, int waves, int columns, float softcap, void* stream) {
+  return nnis_attention_prefill_bf16_more(q, out, k_pages, v_pages, block_table, max_pages, tile_seq, tile_row0, tiles, seq_slot,
+                                          seq_start, seq_pos0, heads, kv_heads, head_dim, window, scale, waves, columns, softcap, 0,
+                                          nullptr, 0, nullptr, stream);
+}
+
 // The sum over the key runs that a call with combine = 0 left in `partial`, for a consumer that does not
 // take the runs as they are.
 extern "C" int nnis_attention_combine(const float* partial, void* out, const int* tok_slot, int tokens, int heads, int head_dim,
@@ -1442,6 +1607,16 @@ extern "C" int nnis_attention_prefill_tile_rows(int, int, int) { return 0; }
 extern "C" int nnis_attention_prefill_max_waves(int, int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
                                            int, const int*, const int*, const int*, int, int, int, int, float, int, int, float, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+}
+extern "C" int nnis_attention_prefill_bf16_more(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                                int, const int*, const int*, const int*, int, int, int, int, float, int, int, float, int,
+                                                const float*, int, const float*, void*) {
+  return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
+}
+extern "C" int nnis_attention_decode_bf16_more(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                               int, int, int, int, int, float, int, int, float*, int, int, int, float, int, const float*,
+                                               int, const float*, void*) {
   return nnis_fail("attention: the matrix-core kernels need keys and values in steps of 16 channels; this module has %d and %d", NNIS_HEAD_DIM, NNIS_VALUE_DIM);
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }

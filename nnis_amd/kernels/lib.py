@@ -102,19 +102,26 @@ def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], r
 
 def _attention_recipe(rest: str) -> ModuleRecipe:
     """``attn_hd<N>``: keys and values of N channels; ``attn_hd<N>v<M>``: values of M; a ``c`` behind either: with a
-    cap of the scores compiled in."""
+    cap of the scores compiled in; an ``x`` at the very end: with the extras of the scores (first keys kept visible
+    beside a window, a bias by distance, a sink in the denominator) compiled into the matrix-core kernels."""
+    name = rest
+    extras = rest.endswith("x")
+    if extras:
+        rest = rest[:-1]
     capped = rest.endswith("c")
     try:
         sizes = [int(part) for part in (rest[:-1] if capped else rest).split("v")]
         if not 1 <= len(sizes) <= 2 or min(sizes) <= 0:
             raise ValueError(rest)
     except ValueError:
-        raise KernelError(f"unknown kernel module 'attn_hd{rest}'") from None
+        raise KernelError(f"unknown kernel module 'attn_hd{name}'") from None
     defines = [("NNIS_HEAD_DIM", str(sizes[0]))]
     if len(sizes) == 2:
         defines.append(("NNIS_VALUE_DIM", str(sizes[1])))
     if capped:
         defines.append(("NNIS_SCORE_CAP", "1"))
+    if extras:
+        defines.append(("NNIS_SCORE_EXTRAS", "1"))
     return ModuleRecipe(("attention.hip",), ("common.h",), tuple(defines), (("attention.hip", tuple(_VECTOR_SUMS)),))
 
 

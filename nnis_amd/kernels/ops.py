@@ -69,6 +69,10 @@ _ATTN_SIGNATURES = {
     "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _VOID],
+    "nnis_attention_prefill_bf16_more": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
+                                         _INT, _INT, _INT, _FLT, _INT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID],
+    "nnis_attention_decode_bf16_more": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
+                                        _INT, _INT, _VOID, _INT, _INT, _INT, _FLT, _INT, _VOID, _INT, _VOID, _VOID],
     "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
                                    _INT, _INT, _VOID, _INT, _INT, _INT, _FLT, _VOID],
@@ -182,15 +186,15 @@ def attention_check(head_dim: int, value_dim: Optional[int] = None) -> None:
         raise Unsupported(f"the attention kernels take values of up to {ATTENTION_MOST_CHANNELS} channels, got {value_dim}")
 
 
-def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0) -> str:
+def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None) -> str:
     """The module compiled for keys of ``head_dim`` channels and values of ``value_dim`` (None: as the keys), with a
-    cap of the scores (``softcap`` > 0) or without."""
+    cap of the scores (``softcap`` > 0) or without, and with the scores' extras (``ScoreExtras``) or without."""
     wide = value_dim is not None and value_dim != head_dim
-    return (f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}") + ("c" if softcap else "")
+    return (f"attn_hd{head_dim}v{value_dim}" if wide else f"attn_hd{head_dim}") + ("c" if softcap else "") + ("x" if extras else "")
 
 
-def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0):
-    name = attention_module_name(head_dim, value_dim, softcap)
+def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None):
+    name = attention_module_name(head_dim, value_dim, softcap, extras)
     if name not in _attn:
         attention_check(head_dim, value_dim)
         _attn[name] = _bind(name, _ATTN_SIGNATURES)
@@ -499,7 +503,7 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
         raise KernelError("attention: key and value pages differ in type")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
         raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
-    lib = attention_module(head_dim, value_dim, softcap)
+    lib = attention_module(head_dim, value_dim, softcap, extras)
     if extras:
         extras.check(heads)
         _check(lib, lib.nnis_attention_rows_more(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
@@ -830,19 +834,20 @@ def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_di
             raise KernelError(f"attention: the matrix-core kernels take bfloat16, {what} is {t.dtype}")
 
 
-def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0) -> int:
+def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None) -> int:
     """Query rows per work item of ``attention_prefill_bf16`` for these sizes.
     ``columns``: the most 16-column tiles (query tiles x heads of a group) a
     wave carries; 0 for as many as the head size allows."""
-    return attention_module(head_dim, value_dim, softcap).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
+    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
 
 
-def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0) -> int:
-    return attention_module(head_dim, value_dim, softcap).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
+def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0, value_dim=None, softcap=0.0, extras=None) -> int:
+    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
 
 
 def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
-                           heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0, value_dim=None, softcap=0.0):
+                           heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0, value_dim=None, softcap=0.0,
+                           extras: Optional[ScoreExtras] = None):
     """Causal attention of whole runs of new tokens over the cache, on the
     matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
     sequence of the step and the first of ``prefill_tile_rows`` rows of its
@@ -855,7 +860,15 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
     tiles = tile_seq.numel()
     if tile_row0.numel() != tiles or seq_start.numel() != seq_slot.numel() + 1 or seq_pos0.numel() != seq_slot.numel():
         raise KernelError("attention: step metadata arrays do not fit each other")
-    lib = attention_module(head_dim, value_dim, softcap)
+    lib = attention_module(head_dim, value_dim, softcap, extras)
+    if extras:
+        extras.check(heads)
+        _check(lib, lib.nnis_attention_prefill_bf16_more(
+            q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+            tile_seq.data_ptr(), tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(), seq_pos0.data_ptr(), heads,
+            kv_heads, head_dim, int(window), float(scale), int(waves), int(columns), float(softcap), extras.keep_first,
+            _ptr(extras.bias), extras.reach, _ptr(extras.sink), _stream()))
+        return out
     _check(lib, lib.nnis_attention_prefill_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
                                                 block_table.data_ptr(), block_table.shape[1], tile_seq.data_ptr(),
                                                 tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(),
@@ -866,7 +879,7 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
                           window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False, token_pages=None,
-                          value_dim=None, softcap=0.0):
+                          value_dim=None, softcap=0.0, extras: Optional[ScoreExtras] = None):
     """One query token per sequence over its cached keys.  The keys are cut
     into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
@@ -897,13 +910,22 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
         if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (value_dim + 4):
             raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (value channels + 4)")
         _dev(partial, "partial")
-    lib = attention_module(head_dim, value_dim, softcap)
-    _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-                                               table.data_ptr(), table.shape[1], tok_slot.data_ptr(),
-                                               tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
-                                               float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
-                                               _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1,
-                                               1 if token_pages is not None else 0, float(softcap), _stream()))
+    lib = attention_module(head_dim, value_dim, softcap, extras)
+    if extras:
+        extras.check(heads)
+        _check(lib, lib.nnis_attention_decode_bf16_more(
+            q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), table.shape[1],
+            tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window), float(scale), int(splits),
+            int(waves), _ptr(partial) if splits > 1 else None, _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1,
+            1 if token_pages is not None else 0, float(softcap), extras.keep_first, _ptr(extras.bias), extras.reach,
+            _ptr(extras.sink), _stream()))
+    else:
+        _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+                                                   table.data_ptr(), table.shape[1], tok_slot.data_ptr(),
+                                                   tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
+                                                   float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
+                                                   _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1,
+                                                   1 if token_pages is not None else 0, float(softcap), _stream()))
     if keep_runs and splits > 1:
         return KeyRuns(partial, int(splits), tokens, heads, value_dim, tok_slot, out, lib)
     return out
@@ -969,8 +991,8 @@ def decode_scratch_held(device):
     return _decode_scratch.get((device.type, device.index))
 
 
-def decode_max_waves(heads: int, kv_heads: int, head_dim: int, value_dim=None, softcap=0.0) -> int:
-    return attention_module(head_dim, value_dim, softcap).nnis_attention_decode_max_waves(heads, kv_heads)
+def decode_max_waves(heads: int, kv_heads: int, head_dim: int, value_dim=None, softcap=0.0, extras=None) -> int:
+    return attention_module(head_dim, value_dim, softcap, extras).nnis_attention_decode_max_waves(heads, kv_heads)
 
 
 def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, width: int = 0):
@@ -1139,24 +1161,25 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     size = max(head_dim, value_dim)  # what a wave's registers are sized by
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if size <= 64 else (2 if size <= 128 else 1)):
         splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * value_dim)
-        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim, value_dim, softcap))
+        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim, value_dim, softcap, extras))
         partial = None
         if splits > 1:
             partial = decode_scratch(q.device, q.shape[0] * heads * splits * (value_dim + 4))
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                                      kv_heads, head_dim, scale, window, splits, partial, waves,
                                      keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS,
-                                     token_pages=tables.pages if tables is not None else None, value_dim=value_dim, softcap=softcap)
+                                     token_pages=tables.pages if tables is not None else None, value_dim=value_dim, softcap=softcap,
+                                     extras=extras)
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
         waves, columns = plan or prefill_plan(ctx.planned_len, ctx.planned_rows, heads, size, kv_heads)
-        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns, value_dim, softcap))
-        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns, value_dim, softcap)
+        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns, value_dim, softcap, extras))
+        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns, value_dim, softcap, extras)
         tiles = ctx.lists.device_list(("attention_tiles", rows), lambda new, first, padded: prefill_tile_list(new, first, padded, rows))
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tiles[0], tiles[1],
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
-                                      waves, columns, value_dim, softcap)
+                                      waves, columns, value_dim, softcap, extras)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window, value_dim, softcap, extras)
 
@@ -1164,7 +1187,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
 def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0,
                               extras: Optional[ScoreExtras] = None) -> bool:
     """Whether ``attention`` takes the matrix-core kernels for these types and sizes (else the 32-bit row kernel)."""
-    return (not extras and q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
+    return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
             and (value_dim or head_dim) % 16 == 0)
 
 

@@ -34,6 +34,11 @@ sets of layer sizes of a real model's kind, each beside a Llama of the same
 width, layers, heads, inner size and vocabulary: a prompt of 2,048 tokens in
 one step and decode at batch 1, 8 and 64, all in one JSON line.
 
+``--workload mutedra`` does the same for the Mutedra design (attention in a
+window with kept first tokens, a bias by distance and a sink; attention over a
+cached latent, plain and with a rotated part, a sink and gates; norms without
+statistics before and after every sublayer).
+
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
 matrix rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
 """
@@ -215,7 +220,8 @@ def prefill_run(shape, rng, tokens=2048):
     del engine
     torch.cuda.empty_cache()
     seconds = sorted(times[3:])[3]  # the median of seven runs of a shape that has come before (and is captured, where it is)
-    flops = (zifunex_step_flops if shape.config.get("architecture") == "Zifunex" else step_flops)(shape.config, [tokens], 1)
+    flops = {"Zifunex": zifunex_step_flops, "Mutedra": mutedra_step_flops}.get(shape.config.get("architecture"), step_flops)(
+        shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
 
@@ -315,13 +321,73 @@ def zifunex_step_flops(config, tokens_per_sequence, wanted_rows):
     return total + 2 * wanted_rows * w * config["vocab"]
 
 
-def zifunex_run(args, rng):
-    """Each set of sizes: the Zifunex model and its Llama twin, a prompt of 2,048 tokens and decode at batch 1, 8, 64."""
+# Mutedra at two sets of layer sizes: W = attention in a window, L = attention over a latent, R = the same with a rotated
+# part, a sink and gates; every layer with a feed-forward; one pass over all layers (its entry adds the pass's vector).
+MUTEDRA_SETS = {
+    "w1024": dict(width=1024, ff=2816, attention=(16, 4, 64, 64), window=(512, 4), bias=(128, 32), latent=(16, 64, 64, 384, 128, 32)),
+    "w2048": dict(width=2048, ff=5632, attention=(16, 4, 128, 128), window=(1024, 4), bias=(128, 32), latent=(16, 128, 128, 768, 192, 64)),
+}
+MUTEDRA_LAYERS = "WLWRWLWR"
+
+
+def mutedra_config(sizes):
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    l_heads, l_dim, l_vdim, q_rank, kv_rank, rot = sizes["latent"]
+    mlp = {"kind": "dense", "ff": sizes["ff"]}
+    kinds = {
+        "W": {"type": "attention", "mlp": mlp, "mixer": {
+            "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "bias_max": sizes["bias"][0],
+            "bias_buckets": sizes["bias"][1], "mask": {"size": sizes["window"][0], "keep_first": sizes["window"][1]}}},
+        "L": {"type": "latent_attention", "mlp": mlp, "mixer": {
+            "heads": l_heads, "dim": l_dim, "vdim": l_vdim, "q_rank": q_rank, "kv_rank": kv_rank, "scale": l_dim ** -0.5}},
+        "R": {"type": "latent_attention_2", "mlp": mlp, "mixer": {
+            "heads": l_heads, "dim": l_dim, "vdim": l_vdim, "q_rank": q_rank, "kv_rank": kv_rank, "scale": (l_dim + rot) ** -0.5,
+            "rot_dim": rot, "rot": {"dims": rot, "base": 10000.0}}},
+    }
+    return {"architecture": "Mutedra", "vocab": ZIFUNEX_VOCAB, "width": sizes["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+            "logit_softcap": 30.0, "layers": [kinds[kind] for kind in MUTEDRA_LAYERS], "loop": {"start": 0, "stop": len(MUTEDRA_LAYERS), "times": 1}}
+
+
+def mutedra_step_flops(config, tokens_per_sequence, wanted_rows):
+    """Multiply-adds x2 of one step over whole prompts from empty slots, as the library computes them (the heads' key
+    and value maps folded into the projections around the latent; a window's keys only as far as it reaches)."""
+    w = config["width"]
+    total = 0
+    for n in tokens_per_sequence:
+        for layer in config["layers"]:
+            m = layer["mixer"]
+            if layer["type"] == "attention":
+                per_token = ((m["heads"] + m["kv_heads"]) * m["dim"] + m["kv_heads"] * m["vdim"]) * w + m["heads"] * m["vdim"] * w
+                reach = m["mask"]["size"] + m["mask"]["keep_first"]
+                keys = n * (n + 1) // 2 if n <= reach else reach * (reach + 1) // 2 + (n - reach) * reach
+                total += 2 * per_token * n + 2 * m["heads"] * (m["dim"] + m["vdim"]) * keys
+            else:
+                rot = m.get("rot_dim", 0)
+                per_token = (m["q_rank"] + m["kv_rank"] + rot) * w + m["heads"] * (m["kv_rank"] + rot) * m["q_rank"] + m["heads"] * m["kv_rank"] * w
+                total += 2 * per_token * n + 2 * m["heads"] * (2 * m["kv_rank"] + rot) * n * (n + 1) // 2
+            if layer["mlp"] is not None:
+                total += 2 * 3 * w * layer["mlp"]["ff"] * n
+    return total + 2 * wanted_rows * w * config["vocab"]
+
+
+def mutedra_twin_config(sizes):
+    """The closest model the library had: a Llama of the same width, layers, inner size and vocabulary, its heads those of
+    the windowed attention."""
+    from nnis_amd.config import preset
+
+    heads, kv_heads, dim, vdim = sizes["attention"]
+    return preset("tinyllama-1.1b", num_hidden_layers=len(MUTEDRA_LAYERS), hidden_size=sizes["width"], num_attention_heads=heads,
+                  num_key_value_heads=kv_heads, head_dim=max(dim, vdim), intermediate_size=sizes["ff"], vocab_size=ZIFUNEX_VOCAB,
+                  max_position_embeddings=ZIFUNEX_CONTEXT, tie_word_embeddings=False)
+
+
+def design_run(args, rng, design, sets, config_of, twin_of):
+    """Each set of sizes: the design's model and its Llama twin, a prompt of 2,048 tokens and decode at batch 1, 8, 64."""
     import torch
 
     out = {}
-    for name, sizes in ZIFUNEX_SETS.items():
-        for which, config in (("zifunex", zifunex_config(sizes)), ("llama", llama_twin_config(sizes))):
+    for name, sizes in sets.items():
+        for which, config in ((design, config_of(sizes)), ("llama", twin_of(sizes))):
             torch.cuda.empty_cache()
             with tempfile.TemporaryDirectory() as folder:
                 shape = Shape(f"{which}-{name}", 0, args.dtype, args.seed, folder, config=config, context=ZIFUNEX_CONTEXT)
@@ -367,7 +433,7 @@ def main() -> int:
     parser.add_argument("--no-other-shapes", action="store_true", help="points of the headline's shape only")
     parser.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     parser.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches (within the context)")
-    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex"], help="run this workload alone")
+    parser.add_argument("--workload", choices=["tinyllama-ragged", "zifunex", "mutedra"], help="run this workload alone")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -377,7 +443,7 @@ def main() -> int:
 
     rng = np.random.default_rng(args.seed)
     if args.workload == "zifunex":
-        models = zifunex_run(args, rng)
+        models = design_run(args, rng, "zifunex", ZIFUNEX_SETS, zifunex_config, llama_twin_config)
         head = models["zifunex-w2048"]["decode_b8"]
         print(json.dumps({
             "metric": "Zifunex at two sets of layer sizes beside a Llama of the same sizes: prefill of 2,048 tokens, decode at batch 1, 8, 64",
@@ -385,6 +451,18 @@ def main() -> int:
             "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights from a seed, uniform-random token ids",
             "config": {"model": "Zifunex, 8 layers of width 2048 (decode at batch 8)", "sets": ZIFUNEX_SETS, "layers": ZIFUNEX_LAYERS,
+                       "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
+            "models": models, "env": environment()}))
+        return 0
+    if args.workload == "mutedra":
+        models = design_run(args, rng, "mutedra", MUTEDRA_SETS, mutedra_config, mutedra_twin_config)
+        head = models["mutedra-w2048"]["decode_b8"]
+        print(json.dumps({
+            "metric": "Mutedra at two sets of layer sizes beside a Llama of the same sizes: prefill of 2,048 tokens, decode at batch 1, 8, 64",
+            "value": head["tokens_per_second"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": head["ms_per_step"], "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights from a seed, uniform-random token ids",
+            "config": {"model": "Mutedra, 8 layers of width 2048 (decode at batch 8)", "sets": MUTEDRA_SETS, "layers": MUTEDRA_LAYERS,
                        "vocab": ZIFUNEX_VOCAB, "context": ZIFUNEX_CONTEXT, "prompt_min": args.prompt_min, "prompt_max": args.prompt_max},
             "models": models, "env": environment()}))
         return 0

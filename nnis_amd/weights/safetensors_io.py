@@ -123,7 +123,7 @@ def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]], me
         if tensor.dtype not in _NAME_OF:
             raise WeightError(f"tensor {name}: dtype {tensor.dtype} cannot be stored")
         t = tensor.detach().cpu().contiguous()
-        raw = t.view(torch.uint8).numpy().tobytes() if t.numel() else b""
+        raw = t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b""  # (a scalar is written as its one element)
         header[name] = {
             "dtype": _NAME_OF[tensor.dtype],
             "shape": list(t.shape),

@@ -40,10 +40,11 @@ constexpr int HD = NNIS_HEAD_DIM;
 #define NNIS_VALUE_DIM NNIS_HEAD_DIM
 #endif
 constexpr int HDV = NNIS_VALUE_DIM;
-// the matrix-core kernels below take heads whose keys and values come in steps of 16 channels
-#define NNIS_MATRIX_CORES (NNIS_HEAD_DIM % 16 == 0 && NNIS_VALUE_DIM % 16 == 0)
 // what a wave's registers are sized by: the larger of the two
 #define NNIS_REG_DIM (NNIS_HEAD_DIM > NNIS_VALUE_DIM ? NNIS_HEAD_DIM : NNIS_VALUE_DIM)
+// the matrix-core kernels below take heads whose keys and values come in steps of 16 channels, up to 256 (beyond, a
+// module holds the row kernel only)
+#define NNIS_MATRIX_CORES (NNIS_HEAD_DIM % 16 == 0 && NNIS_VALUE_DIM % 16 == 0 && NNIS_REG_DIM <= 256)
 constexpr int HDR = NNIS_REG_DIM;
 // 1: scores are bent by a cap before the softmax, s -> cap * tanh(s / cap) (compiled in: the kernels of plain scores stay as they are)
 #ifndef NNIS_SCORE_CAP
@@ -361,6 +362,7 @@ template <int C>
 struct More {
 #if NNIS_SCORE_EXTRAS
   const float* bias_row[C];
+  float far_bias[C];  // the table's last row in the softmax's base-2 units: what every key `reach` and more back gets
   int reach;
   int keep;
 #endif
@@ -377,6 +379,9 @@ __device__ __forceinline__ void attend_block_more(AttnState<C>& st, const QFrag 
   for (int c = 0; c < C; ++c) {
     f32x4 s[2];
     float block_max = -INFINITY;
+    // Most blocks of a long window lie wholly `reach` and more behind every column's query: their keys all read the
+    // table's last row, one number a column, and none needs a look at its distance.
+    const bool far = __all(hi[c] < 0 || hi[c] - (key0 + 31) >= more.reach);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       s[t] = score_tile(f.keys[t], q[c]);
@@ -386,7 +391,8 @@ __device__ __forceinline__ void attend_block_more(AttnState<C>& st, const QFrag 
         const int key = key0 + 8 * g + 4 * t + e;
         const bool seen = key <= hi[c] && (key >= lo[c] || key < more.keep);
         float v = s[t][e] * scale_log2;
-        if (more.bias_row[c] != nullptr && seen) v = fmaf(more.bias_row[c][min(hi[c] - key, more.reach)], kLog2e, v);
+        if (far) v += more.far_bias[c];
+        else if (more.bias_row[c] != nullptr && seen) v = fmaf(more.bias_row[c][min(hi[c] - key, more.reach)], kLog2e, v);
         s[t][e] = seen ? v : -INFINITY;
         block_max = fmaxf(block_max, s[t][e]);
       }
@@ -730,12 +736,14 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   }
   every_lo = __builtin_amdgcn_readfirstlane(every_lo);
   every_hi = __builtin_amdgcn_readfirstlane(every_hi);
-  const int whole_pages = (every_hi + 1) / kPageTokens;  // pages 0 .. whole_pages - 1 of the sequence end at or below every_hi
 #if NNIS_SCORE_EXTRAS
-  const int inner_end = 0;  // (every block goes through the loop that looks at its keys: their distances decide their bias)
-#else
-  const int inner_end = whole_pages > first ? 2 * min(mine, (whole_pages - first + stride - 1) / stride) : 0;  // in blocks of the run
+  // With a bias by distance the blocks that need no look at their keys are those that also lie `reach` and more behind
+  // every column's query: all their keys read the table's last row, one number a column, which the loop without masks
+  // takes as a shift of the column's reference.  (A sink joins the sum at the end and leaves the blocks as they are.)
+  if (a.bias != nullptr) every_hi = every_hi >= 0 ? every_hi - more.reach : -1;
 #endif
+  const int whole_pages = every_hi >= 0 ? (every_hi + 1) / kPageTokens : 0;  // pages 0 .. whole_pages - 1 of the sequence end at or below every_hi
+  const int inner_end = whole_pages > first ? 2 * min(mine, (whole_pages - first + stride - 1) / stride) : 0;  // in blocks of the run
   const int low_page = (every_lo + kPageTokens - 1) / kPageTokens;
   int inner_begin = low_page > first ? 2 * ((low_page - first + stride - 1) / stride) : 0;
   inner_begin = (inner_begin + RING - 1) / RING * RING;  // whole rounds of the ring
@@ -758,6 +766,10 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 #pragma unroll
       for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[0].keys[t], q[0]);
     }
+#if NNIS_SCORE_EXTRAS
+#pragma unroll
+    for (int c = 0; c < C; ++c) st.m[c] -= more.far_bias[c];  // (the reference in the units of scores without their bias; back below)
+#endif
     float rise[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) rise[c] = (st.m[c] + kLazyRise) / a.scale_log2;  // (-inf before a column's first key)
@@ -772,6 +784,10 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
         ask(ring[i], b0 + i + RING);
       }
     }
+#if NNIS_SCORE_EXTRAS
+#pragma unroll
+    for (int c = 0; c < C; ++c) st.m[c] += more.far_bias[c];
+#endif
   }
   // what is left (the diagonal, a short run) one by one
   for (; b0 < blocks; b0 += RING) {
@@ -873,6 +889,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     for (int c = 0; c < C; ++c) {
       const int head = min(head0 + c % GH, a.heads - 1);
       more.bias_row[c] = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
+      more.far_bias[c] = a.bias ? more.bias_row[c][a.reach] * kLog2e : 0.0f;
     }
 #endif
     if (last >= 0) {
@@ -1041,6 +1058,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(Mfma
   for (int c = 0; c < C; ++c) {
     const int head = kv_head * group + (live[c] ? 16 * c + r : 0);
     more.bias_row[c] = a.bias ? a.bias + (size_t)head * (a.reach + 1) : nullptr;
+    more.far_bias[c] = a.bias ? more.bias_row[c][a.reach] * kLog2e : 0.0f;
   }
   // the pages of the kept first keys that lie before the window's first page go with the first run of the keys
   const int kept_pages = split == 0 ? min(page_first, (more.keep + kPageTokens - 1) / kPageTokens) : 0;

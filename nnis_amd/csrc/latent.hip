@@ -109,6 +109,18 @@ __global__ void head_scale_kernel(void* __restrict__ o, int o_dtype, const float
     store_from_f32(o, o_dtype, i, load_as_f32(o, o_dtype, i) * gate[i / channels]);
 }
 
+// the same on bfloat16 rows whose heads come in steps of 8 channels: 16-byte accesses
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_l;
+__global__ void head_scale_bf16_kernel(bf16_t* __restrict__ o, const float* __restrict__ gate, int channels, size_t groups) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += (size_t)gridDim.x * blockDim.x) {
+    const float g = gate[(i * 8) / channels];
+    bf16x8_l v = *(const bf16x8_l*)(o + i * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * g);
+    *(bf16x8_l*)(o + i * 8) = v;
+  }
+}
+
 unsigned blocks_for(size_t total) {
   size_t blocks = (total + 255) / 256;
   return (unsigned)(blocks > 65536 ? 65536 : blocks);
@@ -164,6 +176,12 @@ extern "C" int nnis_head_scale(void* o, int o_dtype, const float* gate, int toke
   NNIS_REQUIRE(o && gate && tokens >= 0 && heads > 0 && channels > 0, "head_scale: bad arguments");
   if (tokens == 0) return 0;
   const size_t total = (size_t)tokens * heads * channels;
+  if (o_dtype == NNIS_BF16 && channels % 8 == 0 && (uintptr_t)o % 16 == 0) {
+    hipLaunchKernelGGL(head_scale_bf16_kernel, dim3(blocks_for(total / 8)), dim3(256), 0, (hipStream_t)stream, (bf16_t*)o, gate, channels,
+                       total / 8);
+    NNIS_LAUNCH_CHECK("head_scale");
+    return 0;
+  }
   hipLaunchKernelGGL(head_scale_kernel, dim3(blocks_for(total)), dim3(256), 0, (hipStream_t)stream, o, o_dtype, gate, channels, total);
   NNIS_LAUNCH_CHECK("head_scale");
   return 0;

@@ -175,15 +175,18 @@ def core():
     return _core
 
 
-ATTENTION_MOST_CHANNELS = 256
+ATTENTION_MOST_CHANNELS = 256  # of the matrix-core kernels
+ATTENTION_ROWS_MOST_CHANNELS = 1024  # of the 32-bit row kernel, which takes what the others do not (a lane's outputs then live in scratch memory)
 
 
-def attention_check(head_dim: int, value_dim: Optional[int] = None) -> None:
-    """Raises ``Unsupported`` for a head size that no attention kernel here takes."""
-    if head_dim <= 0 or head_dim > ATTENTION_MOST_CHANNELS:
-        raise Unsupported(f"the attention kernels take a head_dim up to {ATTENTION_MOST_CHANNELS}, got {head_dim}")
-    if value_dim is not None and value_dim != head_dim and not 0 < value_dim <= ATTENTION_MOST_CHANNELS:
-        raise Unsupported(f"the attention kernels take values of up to {ATTENTION_MOST_CHANNELS} channels, got {value_dim}")
+def attention_check(head_dim: int, value_dim: Optional[int] = None, most: int = ATTENTION_MOST_CHANNELS) -> None:
+    """Raises ``Unsupported`` for a head size that the attention kernels do not take: up to ``most`` channels, by
+    default what the matrix-core kernels carry; a mixer that accepts the row kernel's pace for wider heads asks with
+    ``ATTENTION_ROWS_MOST_CHANNELS``."""
+    if head_dim <= 0 or head_dim > most:
+        raise Unsupported(f"the attention kernels take a head_dim up to {most}, got {head_dim}")
+    if value_dim is not None and value_dim != head_dim and not 0 < value_dim <= most:
+        raise Unsupported(f"the attention kernels take values of up to {most} channels, got {value_dim}")
 
 
 def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None) -> str:
@@ -196,7 +199,7 @@ def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softca
 def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None):
     name = attention_module_name(head_dim, value_dim, softcap, extras)
     if name not in _attn:
-        attention_check(head_dim, value_dim)
+        attention_check(head_dim, value_dim, ATTENTION_ROWS_MOST_CHANNELS)
         _attn[name] = _bind(name, _ATTN_SIGNATURES)
     return _attn[name]
 
@@ -1188,7 +1191,7 @@ def attention_on_matrix_cores(q_dtype, cache_dtype, head_dim: int, value_dim: Op
                               extras: Optional[ScoreExtras] = None) -> bool:
     """Whether ``attention`` takes the matrix-core kernels for these types and sizes (else the 32-bit row kernel)."""
     return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
-            and (value_dim or head_dim) % 16 == 0)
+            and (value_dim or head_dim) % 16 == 0 and max(head_dim, value_dim or head_dim) <= ATTENTION_MOST_CHANNELS)
 
 
 def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, rng: torch.Tensor,

@@ -101,7 +101,8 @@ class LatentAttention(Mixer):
         return KVRequest(1, self.head_width, None, self.kv_rank if self.rot_dim else None)
 
     def check(self, rt):
-        rt.ops.attention_check(self.head_width, self.kv_rank)
+        # (a latent wider than the matrix-core kernels carry still runs, on the row kernel)
+        rt.ops.attention_check(self.head_width, self.kv_rank, rt.ops.ATTENTION_ROWS_MOST_CHANNELS)
 
     def _matrix_cores(self, rt) -> bool:
         return rt.ops.attention_on_matrix_cores(rt.dtype, rt.dtype, self.head_width, self.kv_rank, 0.0, self.extras)

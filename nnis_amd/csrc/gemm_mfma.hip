@@ -88,12 +88,21 @@ constexpr int kFewTokens = NNIS_FEW_TOKENS;
 //   columns of v * v.  The norm's 1 / sqrt(mean + eps) is left to the kernel that reads `scaled`: it needs
 //   the whole row, and the parts of a row are spread over the blocks.  Statistics as in
 //   /root/reference/crates/nnis-model/src/kernels.rs:15-48.
+// With `tanh_norms` the block's norms keep no statistics, N(u) = tanh(alpha u) * w + b, and sit on both sides of the sum:
+//   v = resid + N_post(y);  scaled = bf16(N_next(v)), the next projection's operand as it is;  ss is written and not read.
+// (`gain` is then N_next's weight; all four vectors in gain_dtype.)
 struct ResidualOut {
   float* resid;      // [m, n]
   const void* gain;  // [n], the following norm's weight
   int gain_dtype;
   bf16_t* scaled;    // [m, n]
   float* ss;         // [parts, m]; a part is 16 columns (skinny kernel) or a wave's columns (tiled kernel)
+  int tanh_norms = 0;
+  int tanh_columns = 1;  // n: a flat index's column is index % n
+  const void* next_bias = nullptr;
+  const void* post_weight = nullptr;
+  const void* post_bias = nullptr;
+  float next_alpha = 0.0f, post_alpha = 0.0f;
 };
 
 // four consecutive columns of a token: what the stream and the gain hold there, asked for early.  A gain in
@@ -139,11 +148,23 @@ __device__ __forceinline__ float residual_take(const ResidualOut& o, const Resid
     gain[3] = __uint_as_float(hi & 0xffff0000u);
   }
   bf16x4 scaled;
+  if (o.tanh_norms) {
+    // (the three other vectors are asked for here, behind the main loop: a few words that the caches hold)
+    const int column = (int)(index % (size_t)o.tanh_columns);
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    v[e] += acc[e];
-    if (e < valid) sq = fmaf(v[e], v[e], sq);
-    scaled[e] = (__bf16)(v[e] * gain[e]);
+    for (int e = 0; e < 4; ++e) {
+      const int c = column + (e < valid ? e : 0);
+      const float normed = tanhf(o.post_alpha * acc[e]) * load_as_f32(o.post_weight, o.gain_dtype, c) + load_as_f32(o.post_bias, o.gain_dtype, c);
+      v[e] += normed;
+      scaled[e] = (__bf16)(tanhf(o.next_alpha * v[e]) * gain[e] + load_as_f32(o.next_bias, o.gain_dtype, c));
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] += acc[e];
+      if (e < valid) sq = fmaf(v[e], v[e], sq);
+      scaled[e] = (__bf16)(v[e] * gain[e]);
+    }
   }
   if (valid == 4 && vector_ok) {
     *(f32x4*)(o.resid + index) = v;
@@ -1346,9 +1367,33 @@ extern "C" int nnis_gemm_residual_parts(int m, int n) {
   return n > 16 ? (n + 15) / 16 : 2;
 }
 
+static int gemm_residual_into(const void* x, const void* w, ResidualOut out, int ss_rows, int m, int n, int k, int* parts, int tile_hint,
+                              float* workspace, size_t workspace_bytes, int* pair_count, void* stream_ptr);
+
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
                                   float* ss, int ss_rows, int m, int n, int k, int* parts, int tile_hint, float* workspace,
                                   size_t workspace_bytes, int* pair_count, void* stream_ptr) {
+  ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
+  return gemm_residual_into(x, w, out, ss_rows, m, n, k, parts, tile_hint, workspace, workspace_bytes, pair_count, stream_ptr);
+}
+
+// The same around norms without statistics (see ResidualOut): resid += tanh(post_alpha y) post_weight + post_bias, and
+// `normed` = bf16(tanh(next_alpha resid) next_weight + next_bias), the operand of the projection that follows.
+extern "C" int nnis_gemm_residual_tanh(const void* x, const void* w, float* resid, const void* post_weight, const void* post_bias,
+                                       float post_alpha, const void* next_weight, const void* next_bias, float next_alpha,
+                                       int weights_dtype, void* normed, float* ss, int ss_rows, int m, int n, int k, float* workspace,
+                                       size_t workspace_bytes, int* pair_count, void* stream_ptr) {
+  NNIS_REQUIRE(post_weight && post_bias && next_weight && next_bias, "gemm_residual_tanh: a norm comes with its weight and its bias");
+  ResidualOut out = {resid, next_weight, weights_dtype, (bf16_t*)normed, ss};
+  out.tanh_norms = 1; out.tanh_columns = n; out.next_bias = next_bias; out.post_weight = post_weight; out.post_bias = post_bias;
+  out.next_alpha = next_alpha; out.post_alpha = post_alpha;
+  int parts = 0;
+  return gemm_residual_into(x, w, out, ss_rows, m, n, k, &parts, 0, workspace, workspace_bytes, pair_count, stream_ptr);
+}
+
+static int gemm_residual_into(const void* x, const void* w, ResidualOut out, int ss_rows, int m, int n, int k, int* parts, int tile_hint,
+                              float* workspace, size_t workspace_bytes, int* pair_count, void* stream_ptr) {
+  float* resid = out.resid; const void* gain = out.gain; const int gain_dtype = out.gain_dtype; void* scaled = out.scaled; float* ss = out.ss;
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
   NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual: unknown norm weight dtype %d", gain_dtype);
@@ -1358,7 +1403,6 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   *parts = 0;
   if (m == 0) return 0;
   hipStream_t stream = (hipStream_t)stream_ptr;
-  ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
   NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_residual: the workspace must be 16-byte aligned");
   NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 8), "gemm_residual: unknown tile %d", tile_hint);
   const bool few = tile_hint == 0 && takes_few_tokens_with_parts(m, n, k, workspace != nullptr);  // a tile hint asks for the tiled kernel

@@ -53,6 +53,8 @@ _CORE_SIGNATURES = {
     "nnis_gemm_tile": [_INT, _INT, _INT],
     "nnis_gemm_takes_pair": [_INT, _INT, _INT, _SIZE],
     "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID, _VOID],
+    "nnis_gemm_residual_tanh": [_VOID, _VOID, _VOID, _VOID, _VOID, _FLT, _VOID, _VOID, _FLT, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT,
+                                _VOID, _SIZE, _VOID, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
@@ -781,6 +783,38 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
                                        int(tile), _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0,
                                        work.data_ptr() + GEMM_WORKSPACE_BYTES if work is not None else None, _stream()))
     return parts.value
+
+
+def gemm_residual_tanh(x: torch.Tensor, w, resid: torch.Tensor, post, following, normed: torch.Tensor, ss: torch.Tensor) -> torch.Tensor:
+    """The projection that ends a part of a block whose norms keep no
+    statistics (y -> tanh(alpha y) weight + bias): ``resid`` (float32 [m, n])
+    takes post(x @ w^T) in, in place, and ``normed`` (bfloat16 [m, n]) takes
+    following(resid), the operand of the projection that comes next.
+    ``post`` / ``following``: (alpha, weight, bias).  ``ss``: float32 scratch
+    of ``gemm_residual_parts(m, n)`` rows of m (the kernels' sums of squares,
+    which nobody reads here)."""
+    _packed(w, "gemm_residual_tanh")
+    m, k = x.shape
+    n = w.shape[0]
+    vectors = (post[1], post[2], following[1], following[2])
+    for t, what in ((x, "x"), (resid, "resid"), (normed, "normed"), (ss, "ss")) + tuple((v, "norm vector") for v in vectors):
+        _dev(t, what)
+    if x.dtype != torch.bfloat16 or w.shape[1] != k:
+        raise KernelError("gemm_residual_tanh: x must be bfloat16 [m, k] and the weight bfloat16 [n, k]")
+    if resid.dtype != torch.float32 or tuple(resid.shape) != (m, n) or normed.dtype != torch.bfloat16 or tuple(normed.shape) != (m, n):
+        raise KernelError("gemm_residual_tanh: resid must be float32 [m, n] and normed bfloat16 [m, n]")
+    if any(v.numel() != n or v.dtype != vectors[0].dtype for v in vectors):
+        raise KernelError(f"gemm_residual_tanh: the norms' vectors must have {n} entries of one type")
+    if ss.dtype != torch.float32 or ss.numel() < gemm_residual_parts(m, n) * m:
+        raise KernelError("gemm_residual_tanh: ss must be float32 with gemm_residual_parts(m, n) rows of m")
+    lib = core()
+    work = _gemm_workspace(x.device)
+    _check(lib, lib.nnis_gemm_residual_tanh(x.data_ptr(), w.data_ptr(), resid.data_ptr(), post[1].data_ptr(), post[2].data_ptr(),
+                                            float(post[0]), following[1].data_ptr(), following[2].data_ptr(), float(following[0]),
+                                            _code(vectors[0]), normed.data_ptr(), ss.data_ptr(), ss.numel() // max(m, 1), m, n, k,
+                                            _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0,
+                                            work.data_ptr() + GEMM_WORKSPACE_BYTES if work is not None else None, _stream()))
+    return normed
 
 
 def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, w: torch.Tensor, y: torch.Tensor,

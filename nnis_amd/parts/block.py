@@ -20,7 +20,7 @@ import torch
 from ..errors import InvalidInput
 from ..weights.random_init import register_init_rule
 from .base import Block, TensorSpec, build_part, register_part
-from .lazy import PendingNorm, PostNormed, PreparedRows, PreparedStreams, ResidualInto
+from .lazy import PendingNorm, PostNormed, PreparedRows, PreparedStreams, ResidualInto, TanhInto
 
 
 def _joined(plans):
@@ -254,6 +254,13 @@ class PrePostNormBlock(Block):
         return self.norm1
 
     @staticmethod
+    def _run(part, args, x, post, following, rt):
+        """The part's output, or -- where its last projection took the way out into its own kernel -- ``following``'s rows."""
+        if following is not None and getattr(part, "adds_to_residual", False):
+            return part.forward(*args, into=TanhInto(x, post, following, rt))
+        return part.forward(*args)
+
+    @staticmethod
     def _between(x, y, post, following, rt):
         """x += post(y) in place; returns following(x)."""
         if hasattr(post, "triple") and hasattr(following, "triple"):
@@ -275,12 +282,17 @@ class PrePostNormBlock(Block):
             if isinstance(pending, PostNormed) and not hasattr(self.norm1, "triple"):
                 pending = pending.materialize(rt)
             h = self.norm1.forward(x, rt) if pending is None else self.norm1.add_forward(x, pending, rt)
-        y = self.mixer.forward(h, ctx, view, rt)
+        # A part that ends with a projection may take the way out -- its norm, the sum into the stream, the next norm on
+        # the way in -- into that projection's kernel (``TanhInto``) and then returns the next part's rows, prepared.
+        after_mixer = self.norm2 if self.feed_forward is not None else following
+        y = self._run(self.mixer, (h, ctx, view, rt), x, self.post1, after_mixer, rt)
         post = self.post1
         if self.feed_forward is not None:
-            h = self._between(x, y, self.post1, self.norm2, rt)
-            y = self.feed_forward.forward(h, ctx, rt)
+            h = y.h if isinstance(y, PreparedRows) else self._between(x, y, self.post1, self.norm2, rt)
+            y = self._run(self.feed_forward, (h, ctx, rt), x, self.post2, following, rt)
             post = self.post2
+        if isinstance(y, PreparedRows):
+            return y
         if following is not None and hasattr(post, "triple") and hasattr(following, "triple"):
             return PreparedRows(following, x, self._between(x, y, post, following, rt))
         return x, PostNormed(y, post)

@@ -121,7 +121,9 @@ class LatentAttention(Mixer):
         held = rt.ops.decode_scratch_held(rt.device)
         return [] if held is None else [held]
 
-    def forward(self, x, ctx, view, rt):
+    adds_to_residual = True
+
+    def forward(self, x, ctx, view, rt, into=None):
         tokens = x.shape[0]
         ops = rt.ops
         gates = self.heads if self.gate_name else 0
@@ -147,6 +149,8 @@ class LatentAttention(Mixer):
                               0, tables=step, plan=plan, value_dim=self.kv_rank, extras=self.extras)
         if gates:
             ops.head_scale(mixed, gate, self.heads)
+        if into is not None and into.can_take(mixed, self.out.weight):
+            return into.take(mixed, self.out.weight)  # the output projection adds to the stream itself
         return self.out(mixed, rt)
 
 

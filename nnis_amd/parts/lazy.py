@@ -140,3 +140,35 @@ class PreparedRows:
 
     def __init__(self, norm, x: torch.Tensor, h: torch.Tensor):
         self.norm, self.x, self.h = norm, x, h
+
+
+class TanhInto:
+    """``ResidualInto`` for a block whose norms keep no statistics: where the
+    projection that ends a mixer or feed-forward may put its result.  The
+    stream ``residual`` takes ``post``(product) in, and ``following``, the norm
+    on the next sublayer's way in, is run on the sum, all in the projection's
+    own kernel.  ``take`` returns the ``PreparedRows`` of ``following``."""
+
+    def __init__(self, residual: torch.Tensor, post, following, rt):
+        self.residual, self.post, self.following, self.rt = residual, post, following, rt
+
+    def can_take(self, x, weight) -> bool:
+        residual, rt = self.residual, self.rt
+        return (
+            isinstance(x, torch.Tensor)  # (runs of keys that a decode attention left are added up first)
+            and hasattr(self.post, "triple") and hasattr(self.following, "triple")
+            and rt.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+            and residual.dtype == torch.float32 and residual.is_contiguous()
+            and isinstance(weight, rt.ops.PackedWeight)
+            and weight.shape[0] == residual.shape[1] and weight.shape[1] % 8 == 0
+            and x.data_ptr() % 16 == 0 and residual.data_ptr() % 16 == 0
+            and all(v.data_ptr() % 16 == 0 for v in self.post.triple()[1:] + self.following.triple()[1:])
+        )
+
+    def take(self, x: torch.Tensor, weight) -> PreparedRows:
+        rt, residual = self.rt, self.residual
+        rows, width = residual.shape
+        normed = rt.empty(rows, width)
+        ss = rt.empty(rt.ops.gemm_residual_parts(rows, width), rows, dtype=torch.float32)
+        rt.ops.gemm_residual_tanh(x, weight, residual, self.post.triple(), self.following.triple(), normed, ss)
+        return PreparedRows(self.following, residual, normed)

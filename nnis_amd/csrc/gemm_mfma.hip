@@ -134,6 +134,28 @@ __device__ __forceinline__ ResidualHeld residual_ask(const ResidualOut& o, size_
   return h;
 }
 
+// tanh by the hardware's exponential and reciprocal, 1 - 2 / (e^(2x) + 1): right at both ends (the power overflows to
+// infinity or falls to zero), off by a few 1e-7 in between, which the bfloat16 operand it ends in does not see
+__device__ __forceinline__ float tanh_by_exp2(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.0f);
+}
+
+// four consecutive entries of a vector per column, widened; `whole`: all four exist and lie on an 8- or 16-byte boundary
+__device__ __forceinline__ f32x4 four_of(const void* base, int dtype, int column, int valid, bool whole) {
+  f32x4 out = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (whole) {
+    if (dtype == NNIS_F32) return *(const f32x4*)((const float*)base + column);
+    const uint2 packed = *(const uint2*)((const bf16_t*)base + column);
+    out[0] = __uint_as_float(packed.x << 16);
+    out[1] = __uint_as_float(packed.x & 0xffff0000u);
+    out[2] = __uint_as_float(packed.y << 16);
+    out[3] = __uint_as_float(packed.y & 0xffff0000u);
+    return out;
+  }
+  for (int e = 0; e < valid; ++e) out[e] = load_as_f32(base, dtype, column + e);
+  return out;
+}
+
 // ... and the lane's accumulator acc taken in; returns the lane's part of the row's sum of squares
 __device__ __forceinline__ float residual_take(const ResidualOut& o, const ResidualHeld& h, size_t index, f32x4 acc, int valid,
                                                bool vector_ok) {
@@ -151,12 +173,14 @@ __device__ __forceinline__ float residual_take(const ResidualOut& o, const Resid
   if (o.tanh_norms) {
     // (the three other vectors are asked for here, behind the main loop: a few words that the caches hold)
     const int column = (int)(index % (size_t)o.tanh_columns);
+    const bool whole = valid == 4 && vector_ok;
+    const f32x4 post_w = four_of(o.post_weight, o.gain_dtype, column, valid, whole);
+    const f32x4 post_b = four_of(o.post_bias, o.gain_dtype, column, valid, whole);
+    const f32x4 next_b = four_of(o.next_bias, o.gain_dtype, column, valid, whole);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int c = column + (e < valid ? e : 0);
-      const float normed = tanhf(o.post_alpha * acc[e]) * load_as_f32(o.post_weight, o.gain_dtype, c) + load_as_f32(o.post_bias, o.gain_dtype, c);
-      v[e] += normed;
-      scaled[e] = (__bf16)(tanhf(o.next_alpha * v[e]) * gain[e] + load_as_f32(o.next_bias, o.gain_dtype, c));
+      v[e] += tanh_by_exp2(o.post_alpha * acc[e]) * post_w[e] + post_b[e];
+      scaled[e] = (__bf16)(tanh_by_exp2(o.next_alpha * v[e]) * gain[e] + next_b[e]);
     }
   } else {
 #pragma unroll

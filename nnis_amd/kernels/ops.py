@@ -181,14 +181,19 @@ ATTENTION_MOST_CHANNELS = 256  # of the matrix-core kernels
 ATTENTION_ROWS_MOST_CHANNELS = 1024  # of the 32-bit row kernel, which takes what the others do not (a lane's outputs then live in scratch memory)
 
 
+_wide_heads = set()  # (key channels, value channels) beyond the matrix-core kernels' that a mixer has accepted the row kernel for
+
+
 def attention_check(head_dim: int, value_dim: Optional[int] = None, most: int = ATTENTION_MOST_CHANNELS) -> None:
     """Raises ``Unsupported`` for a head size that the attention kernels do not take: up to ``most`` channels, by
-    default what the matrix-core kernels carry; a mixer that accepts the row kernel's pace for wider heads asks with
-    ``ATTENTION_ROWS_MOST_CHANNELS``."""
+    default what the matrix-core kernels carry.  A mixer that accepts the row kernel's pace for wider heads asks
+    with ``ATTENTION_ROWS_MOST_CHANNELS``; only sizes accepted so are loaded beyond the default."""
     if head_dim <= 0 or head_dim > most:
         raise Unsupported(f"the attention kernels take a head_dim up to {most}, got {head_dim}")
     if value_dim is not None and value_dim != head_dim and not 0 < value_dim <= most:
         raise Unsupported(f"the attention kernels take values of up to {most} channels, got {value_dim}")
+    if most > ATTENTION_MOST_CHANNELS:
+        _wide_heads.add((head_dim, value_dim or head_dim))
 
 
 def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None) -> str:
@@ -201,7 +206,8 @@ def attention_module_name(head_dim: int, value_dim: Optional[int] = None, softca
 def attention_module(head_dim: int, value_dim: Optional[int] = None, softcap: float = 0.0, extras=None):
     name = attention_module_name(head_dim, value_dim, softcap, extras)
     if name not in _attn:
-        attention_check(head_dim, value_dim, ATTENTION_ROWS_MOST_CHANNELS)
+        accepted = (head_dim, value_dim or head_dim) in _wide_heads
+        attention_check(head_dim, value_dim, ATTENTION_ROWS_MOST_CHANNELS if accepted else ATTENTION_MOST_CHANNELS)
         _attn[name] = _bind(name, _ATTN_SIGNATURES)
     return _attn[name]
 

@@ -110,7 +110,8 @@ class LatentAttention(Mixer):
     def decode_plan(self, batch, longest, rt):
         if not self._matrix_cores(rt):
             return None
-        return rt.ops.decode_plan(batch, 1, longest, width=self.heads * self.kv_rank)
+        # (one key/value head makes few blocks: the keys are cut into runs by the rule of narrow outputs, from 9 pages on)
+        return rt.ops.decode_plan(batch, 1, longest, width=min(1024, self.heads * self.kv_rank))
 
     def prompt_plan(self, batch, rows, longest, rt):
         if not self._matrix_cores(rt):

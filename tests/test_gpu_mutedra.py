@@ -112,6 +112,28 @@ def test_the_residual_step_around_a_tanh_norm(y_dtype):
     assert _relative(h.cpu(), M.tanh_norm(y.double(), w[0].double(), w[1].double(), 0.4)) < 1e-6
 
 
+@pytest.mark.parametrize("rows, width, inner", [(1, 64, 96), (8, 256, 384), (16, 100, 72), (200, 256, 640), (2048, 512, 1024), (300, 36, 40)])
+def test_the_way_out_inside_the_projection(rows, width, inner):
+    """The projection that ends a sublayer with the norm on the way out, the sum into the stream and the next norm in its
+    own kernel (few tokens and many, widths that fill no tile) against the three steps one after the other."""
+    from nnis_amd.kernels import ops
+
+    generator = torch.Generator().manual_seed(rows + width)
+    x = torch.randn(rows, inner, generator=generator).to(torch.bfloat16)
+    weight = (torch.randn(width, inner, generator=generator) / inner ** 0.5).to(torch.bfloat16)
+    stream = torch.randn(rows, width, generator=generator)
+    vectors = [torch.randn(width, generator=generator).to(torch.bfloat16) for _ in range(4)]
+    post, following = (1.3, vectors[0].cuda(), vectors[1].cuda()), (0.6, vectors[2].cuda(), vectors[3].cuda())
+    packed = ops.pack_weight(weight.cuda())
+    resid, normed = stream.clone().cuda(), torch.empty(rows, width, device="cuda", dtype=torch.bfloat16)
+    ss = torch.empty(ops.gemm_residual_parts(rows, width), rows, device="cuda")
+    ops.gemm_residual_tanh(x.cuda(), packed, resid, post, following, normed, ss)
+    y = x.double() @ weight.double().T
+    want = stream.double() + M.tanh_norm(y, vectors[0].double(), vectors[1].double(), 1.3)
+    assert _relative(resid.cpu(), want) < 1e-5
+    assert _relative(normed.float().cpu(), M.tanh_norm(want, vectors[2].double(), vectors[3].double(), 0.6)) < 4e-3
+
+
 def test_embedding_scale_logit_cap_and_relu_gate():
     from nnis_amd.kernels import ops
 
@@ -226,7 +248,8 @@ def _latent_part(sizes, width, eps, rotated):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, dim, vdim, q_rank, kv_rank, rot, width", [
-    (3, 16, 24, 40, 32, 16, 64), (2, 24, 8, 16, 48, 0, 48), (2, 32, 32, 24, 64, 32, 96), (5, 8, 40, 48, 40, 0, 40), (4, 24, 16, 32, 24, 8, 56)])
+    (3, 16, 24, 40, 32, 16, 64), (2, 24, 8, 16, 48, 0, 48), (2, 32, 32, 24, 64, 32, 96), (5, 8, 40, 48, 40, 0, 40), (4, 24, 16, 32, 24, 8, 56),
+    (2, 16, 24, 32, 272, 16, 48)])  # (the last: a latent wider than the matrix-core kernels carry runs on the row kernel)
 def test_latent_attention_alone(dtype, heads, dim, vdim, q_rank, kv_rank, rot, width):
     """Attention over the cached latent against the equations, which make every head's keys and values of the latent:
     plain, and with the rotated part, the sink and the gates.  The up projections are large enough for the attention
@@ -238,6 +261,7 @@ def test_latent_attention_alone(dtype, heads, dim, vdim, q_rank, kv_rank, rot, w
     for rope in positions.values():
         rope.bind({}, rt)
         rope.reach(1024)
+    mixer.check(rt)  # (as a model's load does: a latent wider than 256 channels is accepted for the row kernel here)
     mixer.bind(part_w, rt)
     cache = cache_for([mixer.cache_request()], rt, max_tokens=2048, max_positions=1024)
     generator = torch.Generator().manual_seed(5)

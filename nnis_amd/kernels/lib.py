@@ -53,7 +53,7 @@ PREBUILT_HEAD_DIMS = (6, 16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 PREBUILT_WIDE_VALUES = ("attn_hd7v5c", "attn_hd32v16c", "attn_hd16v48c", "attn_hd48v64c", "attn_hd64v32c", "attn_hd6v10c", "attn_hd32c", "attn_hd64c",
                         "attn_hd16c", "attn_hd128c", "attn_hd128v64c",
                         # with the scores' extras (kept first keys, bias by distance, sink), and latents as the one key/value head
-                        "attn_hd32v16x", "attn_hd16v48x", "attn_hd48v32x", "attn_hd96v64x", "attn_hd32v24x", "attn_hd40", "attn_hd288v272x",
+                        "attn_hd32v16x", "attn_hd16v48x", "attn_hd48v32x", "attn_hd96v64x", "attn_hd32v24x", "attn_hd40", "attn_hd288v272x", "attn_hd16x",
                         # the sizes of the measurements of windowed and latent attention
                         "attn_hd64x", "attn_hd128x", "attn_hd160v128x", "attn_hd256v192x")
 

@@ -874,3 +874,108 @@ def test_toy_architecture_with_narrow_values_and_a_sequence_cut_back(tmp_path):
     engine.reset(sb)
     rows = engine.step([StepEntry(sb, a[:9], [8])]).cpu()
     assert_close(rows[0], want_a[8], "float32", "narrow slot reset and used again")
+
+
+# ---------------------------------------------------------------------------
+# a sixth toy architecture: the new block and entry kinds with norms of another
+# kind.  Layers that norm their sublayers on the way in and out with RMS norms
+# (one of them without a feed-forward), an ordinary pre-norm layer behind them,
+# a looped stretch whose passes begin with the embedding added again and a
+# vector of their own, windowed attention with kept first tokens and a sink
+# but no bias: every step between the sublayers is then the norms' own kernel.
+# ---------------------------------------------------------------------------
+def _register_sandwich_toy():
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+
+    @dataclass(frozen=True)
+    class SandwichConfig:
+        width: int
+        vocab_size: int
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["width"], raw["vocab_size"], dict(raw))
+
+    def sandwich_spec(cfg):
+        w = cfg.width
+        rms = lambda name: {"kind": "rms", "width": w, "eps": 1e-5, "weight": name}  # noqa: E731
+        attention = lambda p: {"kind": "causal_attention", "width": w, "heads": 2, "kv_heads": 1, "head_dim": 16, "window": 9,  # noqa: E731
+                               "keep_first": 2, "sink": "zero", "q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}
+        feed = lambda p: {"kind": "gated", "width": w, "inner": 56, "activation": "relu", "gate": p + "g", "up": p + "u", "down": p + "d"}  # noqa: E731
+        layers = [
+            {"kind": "pre_post_norm", "width": w, "norm1": rms("l.0.n1"), "post1": rms("l.0.n1b"), "mixer": attention("l.0."),
+             "norm2": rms("l.0.n2"), "post2": rms("l.0.n2b"), "feed_forward": feed("l.0.")},
+            {"kind": "pre_post_norm", "width": w, "norm1": rms("l.1.n1"), "post1": rms("l.1.n1b"), "mixer": attention("l.1.")},
+            {"kind": "pre_norm", "width": w, "norm1": rms("l.2.n1"), "mixer": dict(attention("l.2."), window=None, keep_first=None, sink=None),
+             "norm2": rms("l.2.n2"), "feed_forward": dict(feed("l.2."), activation="silu")},
+        ]
+        enter = lambda row: {"kind": "restart", "width": w, "table": "passes", "rows": 2, "row": row, "add_embedding": row > 0}  # noqa: E731
+        schedule = [ScheduleEntry(0), ScheduleEntry(1, enter=enter(0)), ScheduleEntry(1, enter=enter(1)), ScheduleEntry(2)]
+        return ModelSpec(
+            architecture="SandwichToyForCausalLM", width=w, vocab_size=cfg.vocab_size, max_positions=256, stored_dtype="bfloat16",
+            embedding={"kind": "table", "vocab_size": cfg.vocab_size, "width": w, "weight": "emb", "scale": 2.0}, positions={},
+            layers=layers, schedule=schedule, final_norm=rms("norm"),
+            head={"kind": "linear", "vocab_size": cfg.vocab_size, "width": w, "weight": "head", "tied_to": None, "softcap": 5.0},
+            config_json=cfg.raw)
+
+    register_architecture("SandwichToyForCausalLM", SandwichConfig, sandwich_spec, replace=True)
+
+
+def _plain_sandwich_toy(folder, ids):
+    from safetensors import safe_open
+
+    with safe_open(folder + "/model.safetensors", framework="pt") as handle:
+        w = {n: handle.get_tensor(n).double() for n in handle.keys()}
+    t = len(ids)
+    norm = lambda x, name: x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w[name]  # noqa: E731
+    place = torch.arange(t)
+
+    def attention(h, p, windowed):
+        q, k, v = (h @ w[p + "q"].T).view(t, 2, 16), h @ w[p + "k"].T, h @ w[p + "v"].T
+        seen = place[None, :] <= place[:, None]
+        if windowed:
+            seen = seen & ((place[:, None] - place[None, :] < 9) | (place[None, :] < 2))
+        out = []
+        for head in range(2):
+            e = torch.where(seen, torch.exp((q[:, head] @ k.T) * 0.25), torch.zeros(t, t, dtype=torch.float64))
+            out.append((e / (e.sum(-1, keepdim=True) + (1.0 if windowed else 0.0))) @ v)
+        return torch.cat(out, dim=-1) @ w[p + "o"].T
+
+    feed = lambda h, p, act: (act(h @ w[p + "g"].T) * (h @ w[p + "u"].T)) @ w[p + "d"].T  # noqa: E731
+    x = w["emb"][torch.tensor(ids)] * 2.0
+    embedded = x.clone()
+    x = x + norm(attention(norm(x, "l.0.n1"), "l.0.", True), "l.0.n1b")
+    x = x + norm(feed(norm(x, "l.0.n2"), "l.0.", torch.relu), "l.0.n2b")
+    for number in range(2):
+        x = x + (embedded if number else 0.0) + w["passes"][number]
+        x = x + norm(attention(norm(x, "l.1.n1"), "l.1.", True), "l.1.n1b")
+    x = x + attention(norm(x, "l.2.n1"), "l.2.", False)
+    x = x + feed(norm(x, "l.2.n2"), "l.2.", torch.nn.functional.silu)
+    z = norm(x, "norm") @ w["head"].T
+    return 5.0 * torch.tanh(z / 5.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_architecture_with_norms_on_both_sides_and_passes(tmp_path, dtype):
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    _register_sandwich_toy()
+    folder = str(tmp_path / "sandwich")
+    raw = {"architectures": ["SandwichToyForCausalLM"], "model_type": "sandwich_toy", "width": 48, "vocab_size": 211}
+    nnis_amd.write_random_model(folder, raw, seed=5)
+    engine = load_engine(folder, dtype=dtype, max_tokens=512)
+    rng = np.random.default_rng(3)
+    a, b = rng.integers(0, 211, size=90).tolist(), rng.integers(0, 211, size=20).tolist()
+    want_a, want_b = _plain_sandwich_toy(folder, a).float(), _plain_sandwich_toy(folder, b).float()
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    rows = engine.step([StepEntry(sa, a[:70], list(range(70))), StepEntry(sb, b[:3], list(range(3)))]).cpu()
+    assert_close(rows[:70], want_a[:70], dtype, "prompt a")
+    assert_close(rows[70:], want_b[:3], dtype, "prompt b")
+    for i in range(17):
+        rows = engine.step([StepEntry(sb, [b[3 + i]], [0]), StepEntry(sa, [a[70 + i]], [0])]).cpu()
+        assert_close(rows[0], want_b[3 + i], dtype, f"decode b {i}")
+        assert_close(rows[1], want_a[70 + i], dtype, f"decode a {i}")

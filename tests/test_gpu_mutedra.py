@@ -321,19 +321,27 @@ def test_a_far_latent_counts(dtype, rot):
 # ---------------------------------------------------------------------------------------------
 
 def _sharpen(folder):
-    """Queries, keys, bias tables, sinks and gates scaled up, so that attention is sharp (a key left out or one too
-    many shows) and every bias row, sink and gate matters."""
+    """A random model's weights are too small for its mixers to matter: their outputs, a few hundredths, would pass the
+    norm on the way out as little more than its bias, and the logits would be the embedding's.  Queries and keys are
+    scaled up so that attention is sharp (a key left out or one too many shows); values, output and feed-forward
+    projections so that every sublayer's output is of order one where its norm bends it; bias tables, sinks, gates and
+    the passes' vectors so that every one of them matters; the head so that the cap bends the logits."""
     path = os.path.join(folder, "model.safetensors")
     tensors = load_file(path)
     for key in tensors:
         if key.endswith((".mix.q", ".mix.k", ".mix.uq", ".mix.uk")):
-            tensors[key] = (tensors[key].float() * 12.0).to(torch.bfloat16)
+            factor = 12.0
+        elif key.endswith((".mix.v", ".mix.o", ".mix.uv", ".mlp.gate", ".mlp.up", ".mlp.down")):
+            factor = 7.0
         elif key.endswith((".mix.rel", ".mix.sink")):
-            tensors[key] = (tensors[key].float() * 80.0).to(torch.bfloat16)
-        elif key.endswith(".mix.g") or key == "loop.step":
-            tensors[key] = (tensors[key].float() * 25.0).to(torch.bfloat16)
+            factor = 80.0
+        elif key.endswith(".mix.g") or key in ("loop.step", "head"):
+            factor = 25.0
         elif key.endswith(".b") or key == "embed":
-            tensors[key] = (tensors[key].float() * 10.0).to(torch.bfloat16)
+            factor = 10.0
+        else:
+            continue
+        tensors[key] = (tensors[key].float() * factor).to(torch.bfloat16)
     save_file(tensors, path)
 
 

@@ -20,17 +20,27 @@ __device__ __forceinline__ float silu_times(float gate, float up) {
   return gate * __builtin_amdgcn_rcpf(1.0f + e) * up;
 }
 
+// The gate's other activations (`act`; 0 is the SiLU above): 1 the tanh form of GELU, 0.5 g (1 + tanh(sqrt(2 / pi) (g +
+// 0.044715 g^3))), its tanh as 1 - 2 / (e^(2x) + 1) by the same two instructions; 2 ReLU, max(g, 0).
+__device__ __forceinline__ float gate_times(float gate, float up, int act) {
+  if (act == 0) return silu_times(gate, up);
+  if (act == 2) return fmaxf(gate, 0.0f) * up;
+  const float inner = 0.7978845608028654f * (gate + 0.044715f * gate * gate * gate);
+  const float tanh_inner = 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(inner * 2.8853900817779268f) + 1.0f);
+  return 0.5f * gate * (1.0f + tanh_inner) * up;
+}
+
 // column: the first of the lane's four channels; inner: channels of the feed-forward
 __device__ __forceinline__ void epilogue_silu(bf16_t* y, int token, int inner, int column, const float (&gate)[4],
-                                              const float (&up)[4]) {
+                                              const float (&up)[4], int act = 0) {
   if (column + 4 <= inner && inner % 4 == 0) {
     epi_bf16x4 packed;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)silu_times(gate[e], up[e]);
+    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)gate_times(gate[e], up[e], act);
     *(epi_bf16x4*)(y + (size_t)token * inner + column) = packed;
   } else {
     for (int e = 0; e < 4; ++e)
-      if (column + e < inner) y[(size_t)token * inner + column + e] = (bf16_t)silu_times(gate[e], up[e]);
+      if (column + e < inner) y[(size_t)token * inner + column + e] = (bf16_t)gate_times(gate[e], up[e], act);
   }
 }
 
@@ -51,6 +61,8 @@ struct RopeTarget {
   const float* tok_cos;
   const float* tok_sin;
   const int* tok_page;
+  // (what the gating epilogue needs rides here too, the one structure that every epilogue is handed)
+  int gate_activation = 0;  // 0 SiLU, 1 tanh-GELU, 2 ReLU: an entry point's `epilogue` argument carries it as 1 + 256 * activation
 };
 
 __device__ __forceinline__ const float* rope_cos_row(const RopeTarget& a, int token, int pos) {

@@ -403,7 +403,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
         hi[e] = acc[1][t][e] * scale;
       }
       if (EPI == EPI_SILU) {
-        epilogue_silu(a.y, token, n / 2, row0 + g * 4, lo, hi);
+        epilogue_silu(a.y, token, n / 2, row0 + g * 4, lo, hi, a.rope.gate_activation);
       } else {
         const int hd = a.rope.head_dim;
         epilogue_rope(a.rope, token, tok_pos[t], tok_page[t], row0 / hd, row0 % hd + g * 4, lo, hi, tok_cos[t], tok_sin[t]);
@@ -457,6 +457,11 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, f
               hipStream_t stream) {
   const int n = a.n, k = a.k;
   a.stream_weights = (size_t)n * k * sizeof(bf16_t) > kStreamWeightBytes;
+  if ((epilogue & 0xff) == EPI_SILU) {  // the gate's activation rides in the bits above
+    a.rope.gate_activation = epilogue >> 8;
+    NNIS_REQUIRE(a.rope.gate_activation >= 0 && a.rope.gate_activation <= 2, "gemm_fused: unknown gate activation %d", a.rope.gate_activation);
+    epilogue = EPI_SILU;
+  }
   int units;
   if (epilogue == EPI_STORE) {
     units = (n + 15) / 16;

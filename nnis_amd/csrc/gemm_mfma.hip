@@ -876,7 +876,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t
           hi[e] = acc[i][2 * u + 1][e] * scale;
         }
         if constexpr (EPI == EPI_SILU) {
-          epilogue_silu(y.y, token, n / 2, first + 4 * g, lo, hi);
+          epilogue_silu(y.y, token, n / 2, first + 4 * g, lo, hi, y.rope.gate_activation);
         } else {
           const int hd = y.rope.head_dim, head = first / hd, f0 = first % hd + 4 * g;
           epi_f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1015,7 +1015,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
     if (rest_lo > 0) store4(y.y, (size_t)token * n + column, (f32x4){lo[0], lo[1], lo[2], lo[3]}, rest_lo >= 4 ? 4 : rest_lo, vector_ok);
     if (rest_hi > 0) store4(y.y, (size_t)token * n + column + 16, (f32x4){hi[0], hi[1], hi[2], hi[3]}, rest_hi >= 4 ? 4 : rest_hi, vector_ok);
   } else if constexpr (EPI == EPI_SILU) {
-    if (unit * 16 < n / 2) epilogue_silu(y.y, token, n / 2, unit * 16 + quad * 4, lo, hi);
+    if (unit * 16 < n / 2) epilogue_silu(y.y, token, n / 2, unit * 16 + quad * 4, lo, hi, y.rope.gate_activation);
   } else {
     const int hd = y.rope.head_dim, per_head = hd / 32;
     if (unit >= (y.rope.heads + 2 * y.rope.kv_heads) * per_head) return;

@@ -659,6 +659,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, split: int = 
 
 
 EPILOGUE_STORE, EPILOGUE_SILU, EPILOGUE_ROPE = 0, 1, 2
+# the gating epilogue with another activation than SiLU: the activation's code (``ACTIVATIONS``) rides above the epilogue's
+EPILOGUE_GATE = {"silu": EPILOGUE_SILU, "gelu_tanh": EPILOGUE_SILU + 256 * 1, "relu": EPILOGUE_SILU + 256 * 2}
 FUSED_MAX_TOKENS = 16  # beyond a tile of 16 tokens every wave re-reads too much of x: the separate kernels win
 
 
@@ -705,7 +707,9 @@ def _step_table_pointers(rope: dict):
 
 def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, rope: Optional[dict]) -> dict:
     """Checks y and the rotating epilogue's arguments against the sizes; returns the arguments (or {})."""
-    expect = {EPILOGUE_STORE: (m, n), EPILOGUE_SILU: (m, n // 2)}.get(epilogue)
+    expect = {EPILOGUE_STORE: (m, n), EPILOGUE_SILU: (m, n // 2)}.get(epilogue & 0xff if epilogue > 0 else epilogue)
+    if epilogue >> 8 and ((epilogue & 0xff) != EPILOGUE_SILU or epilogue >> 8 not in ACTIVATIONS.values()):
+        raise KernelError(f"{what}: unknown epilogue {epilogue}")
     r = rope or {}
     if epilogue == EPILOGUE_ROPE:
         expect = (m, r["heads"] * r["head_dim"])
@@ -848,6 +852,33 @@ def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, 
         r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), *_step_table_pointers(r), int(split), _ptr(work),
         GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return y
+
+
+_unit_rows = {}  # per device: zeros that stand for rows whose scale is one
+UNIT_ROWS_MOST = 1 << 16
+
+
+def gated_linear(x: torch.Tensor, weight, out: torch.Tensor, activation: str) -> torch.Tensor:
+    """out = act(x @ gate^T) * (x @ up^T) for a packed weight whose first half
+    of rows is the gate: the product with the gating in its epilogue, on plain
+    rows (``gemm_scaled`` with a row scale of one: sums of squares of zero and
+    an eps of one).  Up to ``UNIT_ROWS_MOST`` rows; call ``unit_rows(device)``
+    once outside any graph capture before the first use."""
+    m = x.shape[0]
+    if m > UNIT_ROWS_MOST:
+        raise KernelError(f"gated_linear: up to {UNIT_ROWS_MOST} rows are taken, got {m}")
+    return gemm_scaled(x, unit_rows(x.device)[:m].view(1, m), 1, 1.0, weight, out, EPILOGUE_GATE[activation])
+
+
+def unit_rows(device) -> torch.Tensor:
+    device = torch.device(device)
+    key = (device.type, device.index)
+    held = _unit_rows.get(key)
+    if held is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("gated_linear: its rows of zeros would have to be made inside a graph capture")
+        held = _unit_rows[key] = torch.zeros(UNIT_ROWS_MOST, dtype=torch.float32, device=device)
+    return held
 
 
 def linear(x: torch.Tensor, weight, out: torch.Tensor) -> torch.Tensor:

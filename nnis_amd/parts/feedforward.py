@@ -33,6 +33,8 @@ class GatedFeedForward(FeedForward):
         ]
 
     def bind(self, weights, rt):
+        if rt.dtype == torch.bfloat16:
+            rt.ops.unit_rows(rt.device)  # (made here, outside any captured step)
         self.gate_up = Projection(torch.cat([weights[self.names["gate"]], weights[self.names["up"]]], dim=0), rt)
         self.down = Projection(weights[self.names["down"]], rt)
 
@@ -51,8 +53,14 @@ class GatedFeedForward(FeedForward):
         else:
             if isinstance(x, PendingNorm):
                 x = x.materialize()
-            gate_up = self.gate_up(x, rt)
-            hidden = rt.ops.gated_act(gate_up, rt.empty(x.shape[0], self.inner), self.activation)
+            ops = rt.ops
+            if (rt.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and isinstance(self.gate_up.weight, ops.PackedWeight)
+                    and 0 < x.shape[0] <= ops.UNIT_ROWS_MOST and x.is_contiguous() and x.data_ptr() % 16 == 0):
+                # both projections with the gating in their epilogue, on rows that are normed already
+                hidden = ops.gated_linear(x, self.gate_up.weight, rt.empty(x.shape[0], self.inner), self.activation)
+            else:
+                gate_up = self.gate_up(x, rt)
+                hidden = ops.gated_act(gate_up, rt.empty(x.shape[0], self.inner), self.activation)
         if into is not None and into.can_take(hidden, self.down.weight):
             return into.take(hidden, self.down.weight)  # the down projection adds to the stream itself
         return self.down(hidden, rt)

@@ -134,6 +134,22 @@ def test_the_way_out_inside_the_projection(rows, width, inner):
     assert _relative(normed.float().cpu(), M.tanh_norm(want, vectors[2].double(), vectors[3].double(), 0.6)) < 4e-3
 
 
+@pytest.mark.parametrize("activation", ["relu", "gelu_tanh", "silu"])
+@pytest.mark.parametrize("rows, width, inner", [(1, 64, 96), (8, 256, 384), (40, 128, 200), (200, 256, 640), (2048, 512, 1024), (300, 40, 36)])
+def test_the_gate_inside_the_projection(activation, rows, width, inner):
+    """Gate and up projection with the gating in the product's epilogue, on plain rows, against the products in 64-bit."""
+    from nnis_amd.kernels import ops
+
+    generator = torch.Generator().manual_seed(rows + inner)
+    x = torch.randn(rows, width, generator=generator).to(torch.bfloat16)
+    weight = (3.0 * torch.randn(2 * inner, width, generator=generator) / width ** 0.5).to(torch.bfloat16)
+    got = ops.gated_linear(x.cuda(), ops.pack_weight(weight.cuda()), torch.empty(rows, inner, device="cuda", dtype=torch.bfloat16), activation)
+    gate, up = x.double() @ weight[:inner].double().T, x.double() @ weight[inner:].double().T
+    act = {"relu": torch.relu, "silu": torch.nn.functional.silu,
+           "gelu_tanh": lambda g: 0.5 * g * (1 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))}[activation]
+    assert _relative(got.float().cpu(), act(gate) * up) < 4e-3
+
+
 def test_embedding_scale_logit_cap_and_relu_gate():
     from nnis_amd.kernels import ops
 

@@ -4,8 +4,13 @@ A Mutedra folder names its design in ``architecture`` and gives every size and
 constant that may differ between models: ``vocab``, ``width``, ``norm.eps``,
 ``embedding.scale``, ``logit_softcap``, ``layers`` (each with ``type``, the
 mixer's sizes in ``mixer`` and ``mlp`` -- ``{"kind": "dense", "ff": n}`` or
-null) and ``loop`` (``start``, ``stop``, ``times``).  Nothing has a default: a
-key that is missing is an error, so that a model never runs on a guess.  One
+null) and ``loop`` (``start``, ``stop``, ``times``).  No size has a default: a
+size that is missing is an error, so that a model never runs on a guess.  A
+mechanism that the file does not mention at all does not exist in that model:
+without ``loop`` no layer runs twice and no pass begins, without
+``embedding.scale`` or ``logit_softcap`` rows and logits stay as they are,
+an ``attention`` mixer without ``mask`` sees every earlier key and without
+``bias_max`` has no bias by distance.  One
 size is not in the file, the number of rows of an ``attention`` mixer's table
 of distance biases; it is read from the tensor (a configuration written for a
 random model names it as ``bias_buckets``).
@@ -33,17 +38,19 @@ class WindowedSizes:
     dim: int
     vdim: int
     scale: float
-    window: int
+    window: int  # 0: no window, every earlier key is seen
     keep_first: int
-    bias_max: int
+    bias_max: int  # 0: no bias by distance
     bias_buckets: Optional[int]
 
     @classmethod
     def from_dict(cls, raw, where):
-        mask = _get(raw, "mask", where)
+        mask = raw.get("mask") if isinstance(raw, dict) else None
+        biased = isinstance(raw, dict) and raw.get("bias_max") is not None
         out = cls(_int(raw, "heads", where), _int(raw, "kv_heads", where), _int(raw, "dim", where), _int(raw, "vdim", where),
-                  _number(raw, "scale", where), _int(mask, "size", where + ".mask"),
-                  _int(mask, "keep_first", where + ".mask", least=0), _int(raw, "bias_max", where, least=2),
+                  _number(raw, "scale", where), _int(mask, "size", where + ".mask") if mask is not None else 0,
+                  _int(mask, "keep_first", where + ".mask", least=0) if mask is not None else 0,
+                  _int(raw, "bias_max", where, least=2) if biased else 0,
                   _int(raw, "bias_buckets", where, least=2) if "bias_buckets" in raw else None)
         if out.heads % out.kv_heads:
             raise InvalidInput(f"config.json {where}: {out.heads} heads do not divide into {out.kv_heads} kv_heads")
@@ -121,15 +128,18 @@ class MutedraConfig:
                 out_layers.append(LayerSizes(kind, latent=LatentSizes.from_dict(mixer, where + ".mixer", kind.endswith("_2")), ff=ff))
             else:
                 raise Unsupported(f"config.json {where}.type {kind!r}; this design has the mixers {', '.join(MIXERS)}")
-        loop = _get(raw, "loop", "file")
-        start, stop = _int(loop, "start", "loop", least=0), _int(loop, "stop", "loop", least=0)
-        times = _int(loop, "times", "loop", least=1)
-        if not start <= stop <= len(out_layers):
-            raise InvalidInput(f"config.json loop covers layers {start} to {stop - 1}, but there are {len(out_layers)}")
+        loop = raw.get("loop")
+        start, stop, times = 0, 0, 1
+        if loop is not None:
+            start, stop = _int(loop, "start", "loop", least=0), _int(loop, "stop", "loop", least=0)
+            times = _int(loop, "times", "loop", least=1)
+            if not start <= stop <= len(out_layers):
+                raise InvalidInput(f"config.json loop covers layers {start} to {stop - 1}, but there are {len(out_layers)}")
+        embedding = raw.get("embedding") or {}
         return cls(
             vocab=_int(raw, "vocab", "file"), width=_int(raw, "width", "file"), eps=_number(_get(raw, "norm", "file"), "eps", "norm"),
-            embedding_scale=_number(_get(raw, "embedding", "file"), "scale", "embedding"),
-            logit_softcap=_number(raw, "logit_softcap", "file"), layers=out_layers, loop_start=start, loop_stop=stop,
+            embedding_scale=_number(embedding, "scale", "embedding") if embedding.get("scale") is not None else 1.0,
+            logit_softcap=_number(raw, "logit_softcap", "file") if raw.get("logit_softcap") is not None else 0.0, layers=out_layers, loop_start=start, loop_stop=stop,
             loop_times=times, raw=copy.deepcopy(raw))
 
     def layer_runs(self):

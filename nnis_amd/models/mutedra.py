@@ -23,12 +23,16 @@ def _norm(cfg: MutedraConfig, name: str):
 
 
 def _windowed(cfg: MutedraConfig, prefix: str, sizes):
-    return {
+    out = {
         "kind": "causal_attention", "width": cfg.width, "heads": sizes.heads, "kv_heads": sizes.kv_heads, "head_dim": sizes.dim,
-        "value_dim": sizes.vdim, "scale": sizes.scale, "window": sizes.window, "keep_first": sizes.keep_first,
-        "distance_bias": prefix + "rel", "bias_reach": sizes.bias_max, "bias_buckets": sizes.bias_buckets, "sink": "zero",
+        "value_dim": sizes.vdim, "scale": sizes.scale, "sink": "zero",
         "q": prefix + "q", "k": prefix + "k", "v": prefix + "v", "o": prefix + "o",
     }
+    if sizes.window:
+        out.update(window=sizes.window, keep_first=sizes.keep_first)
+    if sizes.bias_max:
+        out.update(distance_bias=prefix + "rel", bias_reach=sizes.bias_max, bias_buckets=sizes.bias_buckets)
+    return out
 
 
 def _latent(cfg: MutedraConfig, prefix: str, sizes, position):
@@ -81,7 +85,7 @@ def mutedra_spec(cfg: MutedraConfig) -> ModelSpec:
         schedule=schedule,
         final_norm=_norm(cfg, "final.norm"),
         head={"kind": "linear", "vocab_size": cfg.vocab, "width": cfg.width, "weight": "head", "tied_to": None,
-              "softcap": cfg.logit_softcap},
+              "softcap": cfg.logit_softcap or None},
         stop_token_ids=(),
         config_json=cfg.to_dict(),
     )

@@ -41,17 +41,21 @@ def windowed_attention(h, w, sizes, rnd=identity):
     q . k * scale + rel[row(i - j), head]; the weights are exp(s) / (1 + sum exp(s))."""
     n = h.shape[0]
     heads, groups, dim, vdim = sizes["heads"], sizes["kv_heads"], sizes["dim"], sizes["vdim"]
-    window, keep = sizes["mask"]["size"], sizes["mask"]["keep_first"]
+    mask = sizes.get("mask")  # (without one every earlier key is seen; without bias_max there is no bias)
+    window, keep = (mask["size"], mask["keep_first"]) if mask else (n, 0)
     q = rnd(h @ w["q"].T).view(n, heads, dim)
     k = rnd(h @ w["k"].T).view(n, groups, dim)
     v = rnd(h @ w["v"].T).view(n, groups, vdim)
-    rows = torch.tensor([bias_row(d, w["rel"].shape[0], sizes["bias_max"]) for d in range(n)])
+    biased = sizes.get("bias_max") is not None
+    rows = torch.tensor([bias_row(d, w["rel"].shape[0], sizes["bias_max"]) if biased else 0 for d in range(n)])
     i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
     seen = (j <= i) & ((i - j < window) | (j < keep))
     out = torch.zeros(n, heads, vdim, dtype=torch.float64)
     for head in range(heads):
         group = head // (heads // groups)
-        s = (q[:, head] @ k[:, group].T) * sizes["scale"] + w["rel"][rows[(i - j).clamp(min=0)], head]
+        s = (q[:, head] @ k[:, group].T) * sizes["scale"]
+        if biased:
+            s = s + w["rel"][rows[(i - j).clamp(min=0)], head]
         s = torch.where(seen, s, torch.full_like(s, -math.inf))
         top = s.max(dim=1, keepdim=True).values.clamp(min=0.0)  # the sink's score is 0
         e = torch.exp(s - top)
@@ -128,7 +132,8 @@ class PlainMutedra:
 
     def runs(self):
         """[(layer, number of the pass that begins there or None)]"""
-        loop, count = self.config["loop"], len(self.config["layers"])
+        count = len(self.config["layers"])
+        loop = self.config.get("loop") or {"start": 0, "stop": 0, "times": 1}
         out = [(i, None) for i in range(loop["start"])]
         for number in range(loop["times"]):
             out += [(i, number if i == loop["start"] else None) for i in range(loop["start"], loop["stop"])]
@@ -136,7 +141,7 @@ class PlainMutedra:
 
     def logits(self, ids, rnd=identity, stream_after=None):
         cfg = self.config
-        x = self.w["embed"][torch.tensor(list(ids))] * cfg["embedding"]["scale"]
+        x = self.w["embed"][torch.tensor(list(ids))] * (cfg.get("embedding") or {}).get("scale", 1.0)
         embedded = x.clone()
         for index, number in self.runs():
             if number is not None:
@@ -156,7 +161,8 @@ class PlainMutedra:
             if stream_after is not None:
                 stream_after.append(x.clone())
         z = rnd(self._norm(x, "final.norm")) @ self.w["head"].T
-        return cfg["logit_softcap"] * torch.tanh(z / cfg["logit_softcap"])
+        cap = cfg.get("logit_softcap")
+        return z if cap is None else cap * torch.tanh(z / cap)
 
     def greedy(self, ids, count):
         ids, out = list(ids), []

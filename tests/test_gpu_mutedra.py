@@ -540,6 +540,25 @@ def test_the_command_line_runs_the_model(folders):
     assert [int(t) for t in done.stdout.strip().splitlines()[-1].split(",")] == plain.greedy([5, 17, 3], 4)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_model_without_the_optional_mechanisms(tmp_path, dtype):
+    """No loop, no embedding scale, no cap of the logits, an attention without window and bias (the sink stays)."""
+    import copy
+
+    config = copy.deepcopy(MUTEDRA_CONFIGS["A"][0])
+    del config["loop"], config["logit_softcap"], config["embedding"]["scale"]
+    del config["layers"][1]["mixer"]["mask"], config["layers"][1]["mixer"]["bias_max"], config["layers"][1]["mixer"]["bias_buckets"]
+    folder = str(tmp_path / "bare")
+    nnis_amd.write_random_model(folder, config, 41)
+    _sharpen(folder)
+    plain = M.PlainMutedra(folder)
+    engine = nnis_amd.load_engine(folder, dtype=dtype, max_tokens=512)
+    ids = _ids(100, config["vocab"], 6)
+    slot = engine.start_sequence()
+    got = _collect(engine, slot, ids, [70] + list(range(71, 101)))
+    Yardstick(plain).check(got, ids, dtype, "a model without the optional mechanisms")
+
+
 SIZES = {"attention": [(32, 16), (16, 48)], "latent": [(32, 16), (48, 0), (64, 32), (40, 0), (24, 8)]}  # modules that are built beforehand
 
 

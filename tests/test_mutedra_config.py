@@ -45,9 +45,9 @@ def test_passes_and_their_entries(config, runs):
 
 
 def test_missing_and_wrong_keys_are_refused():
-    for path in (["vocab"], ["norm", "eps"], ["embedding", "scale"], ["logit_softcap"], ["loop"], ["loop", "times"],
+    for path in (["vocab"], ["norm", "eps"], ["loop", "times"],
                  ["layers", 0, "mixer", "kv_rank"], ["layers", 0, "mixer", "rot"], ["layers", 0, "mixer", "rot_dim"],
-                 ["layers", 1, "mixer", "mask"], ["layers", 1, "mixer", "mask", "keep_first"], ["layers", 1, "mixer", "bias_max"],
+                 ["layers", 1, "mixer", "mask", "keep_first"], ["layers", 1, "mixer", "scale"],
                  ["layers", 1, "mlp"], ["layers", 2, "mlp", "ff"], ["layers", 2, "mixer", "q_rank"]):
         raw = copy.deepcopy(MUT_A)
         at = raw
@@ -65,6 +65,21 @@ def test_missing_and_wrong_keys_are_refused():
         change(raw)
         with pytest.raises(error):
             spec_from_config(raw)
+
+
+def test_a_mechanism_that_the_file_does_not_mention_does_not_exist():
+    raw = copy.deepcopy(MUT_A)
+    del raw["loop"], raw["logit_softcap"], raw["embedding"]["scale"]
+    del raw["layers"][1]["mixer"]["mask"], raw["layers"][1]["mixer"]["bias_max"]
+    cfg, spec = spec_from_config(raw)
+    assert cfg.layer_runs() == [(0, None), (1, None), (2, None)] and all(entry.enter is None for entry in spec.schedule)
+    assert spec.embedding["scale"] == 1.0 and spec.head["softcap"] is None
+    mixer = spec.layers[1]["mixer"]
+    assert "window" not in mixer and "distance_bias" not in mixer and mixer["sink"] == "zero"
+    model = DecoderModel(spec)
+    names = {t.name for t in model.tensors()}
+    assert "loop.step" not in names and "l1.mix.rel" not in names
+    assert model.cache_requests()[0][1][1] == KVRequest(2, 32, None, 16)
 
 
 def test_tensors_and_cache_requests():
